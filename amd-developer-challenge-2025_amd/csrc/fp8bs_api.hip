@@ -1,0 +1,184 @@
+// C ABI of libfp8bs.so (declared in include/fp8bs.h): argument checking, the shape-family planner
+// and kernel launches.  Host code only; the device code is in fp8bs_kernels.hip.
+//
+// This layer stands where the reference has its launcher `fp8_mm(...)`
+// (1-amd-fp8-mm/amd-fp8-mm-submission.py:514-579).  Differences by design: it is stream-aware,
+// returns a status instead of void, never writes the inputs, and picks kernels by shape family
+// instead of an exact-shape table.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "fp8bs.h"
+#include "fp8bs_kernels.h"
+
+namespace {
+
+constexpr int KBLK = 128;
+
+struct VariantInfo { int bm, bn, threads; };
+
+bool variant_info(int variant, VariantInfo* out) {
+    switch (variant) {
+        case FP8BS_VARIANT_GENERIC:  *out = {16, 16, 256}; return true;
+        case FP8BS_VARIANT_T256x256: *out = {256, 256, 512}; return true;
+        case FP8BS_VARIANT_T128x128: *out = {128, 128, 256}; return true;
+        case FP8BS_VARIANT_T64x128:  *out = {64, 128, 256}; return true;
+        case FP8BS_VARIANT_T256x128: *out = {256, 128, 512}; return true;
+        default: return false;
+    }
+}
+
+inline long cdiv(long a, long b) { return (a + b - 1) / b; }
+
+// Fill a plan for a given variant and split count.
+void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out) {
+    VariantInfo vi{};
+    variant_info(variant, &vi);
+    int kbt = k / KBLK;
+    if (variant == FP8BS_VARIANT_GENERIC) split_k = 1;
+    if (split_k < 1) split_k = 1;
+    if (split_k > kbt) split_k = kbt > 0 ? kbt : 1;
+    out->variant = variant;
+    out->tile_m = vi.bm;
+    out->tile_n = vi.bn;
+    out->split_k = split_k;
+    out->block_threads = vi.threads;
+    out->lds_bytes = fp8bs::variant_lds_bytes(variant);
+    out->reserved = 0;
+    if (variant == FP8BS_VARIANT_GENERIC) {
+        out->grid_x = (int)cdiv(n, 16); out->grid_y = (int)cdiv(m, 16); out->grid_z = 1;
+    } else {
+        out->grid_x = (int)(cdiv(m, vi.bm) * cdiv(n, vi.bn) * split_k); out->grid_y = 1; out->grid_z = 1;
+    }
+    out->workspace_bytes = split_k > 1 ? (uint64_t)split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
+}
+
+// Shape-family rule.  m or n not a multiple of 16 -> generic kernel (the tiled kernels copy 16-byte
+// chunks along m and n).  Otherwise pick the largest tile that still fills the chip, and split K when
+// even the smallest tile leaves most CUs idle (skinny-M, bandwidth-bound shapes).
+void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
+    if (num_cus <= 0) num_cus = 256;
+    if ((m % 16) != 0 || (n % 16) != 0) { fill_plan(m, n, k, FP8BS_VARIANT_GENERIC, 1, out); return; }
+    int kbt = k / KBLK;
+    long t256 = cdiv(m, 256) * cdiv(n, 256);
+    long t128 = cdiv(m, 128) * cdiv(n, 128);
+    if (m > 64 && t256 * 10 >= (long)num_cus * 9) { fill_plan(m, n, k, FP8BS_VARIANT_T256x256, 1, out); return; }
+    if (m > 64 && t128 >= num_cus) { fill_plan(m, n, k, FP8BS_VARIANT_T128x128, 1, out); return; }
+    int variant = m <= 64 ? FP8BS_VARIANT_T64x128 : FP8BS_VARIANT_T128x128;
+    VariantInfo vi{};
+    variant_info(variant, &vi);
+    long tiles = cdiv(m, vi.bm) * cdiv(n, vi.bn);
+    // aim for about two workgroups per CU, keep at least 4 K blocks per split
+    long want = cdiv(2L * num_cus, tiles);
+    long max_split = kbt / 4 > 0 ? kbt / 4 : 1;
+    long s = want < 1 ? 1 : (want > max_split ? max_split : want);
+    if (s > 16) s = 16;
+    fill_plan(m, n, k, variant, (int)s, out);
+}
+
+int check_common(const void* a, const void* b, const float* as, const float* bs, void* c, int m, int n, int k) {
+    if (m < 0 || n < 0 || k < 0 || (k % KBLK) != 0) return FP8BS_ERR_BAD_SHAPE;
+    if (m == 0 || n == 0) return FP8BS_OK;   // nothing to write
+    if (!a || !b || !as || !bs || !c) {
+        if (k == 0 && c) return FP8BS_OK;
+        return FP8BS_ERR_NULL_POINTER;
+    }
+    if ((uint64_t)m * (uint64_t)k >= (1ull << 32) || (uint64_t)n * (uint64_t)k >= (1ull << 32)) return FP8BS_ERR_TOO_LARGE;
+    return FP8BS_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fp8bs_version(void) { return 100; }
+
+const char* fp8bs_strerror(int status) {
+    switch (status) {
+        case FP8BS_OK: return "success";
+        case FP8BS_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case FP8BS_ERR_BAD_SHAPE: return "bad shape: m, n, k must be non-negative and k a multiple of 128";
+        case FP8BS_ERR_WORKSPACE: return "workspace missing or smaller than fp8bs_workspace_bytes()";
+        case FP8BS_ERR_TOO_LARGE: return "operand exceeds the 4 GiB buffer-addressing limit (m*k or n*k >= 2^32)";
+        case FP8BS_ERR_LAUNCH: return "kernel launch failed";
+        case FP8BS_ERR_BAD_OFFSETS: return "grouped: num_experts must be positive";
+        case FP8BS_ERR_BAD_VARIANT: return "unknown or inapplicable kernel variant";
+        default: return "unknown fp8bs status";
+    }
+}
+
+int fp8bs_plan(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
+    if (!out) return FP8BS_ERR_NULL_POINTER;
+    if (m <= 0 || n <= 0 || k <= 0 || (k % KBLK) != 0) return FP8BS_ERR_BAD_SHAPE;
+    choose(m, n, k, num_cus, out);
+    return FP8BS_OK;
+}
+
+size_t fp8bs_workspace_bytes(int m, int n, int k) {
+    fp8bs_plan_t p{};
+    if (fp8bs_plan(m, n, k, 0, &p) != FP8BS_OK) return 0;
+    return (size_t)p.workspace_bytes;
+}
+
+int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                  void* c, void* ws, size_t ws_bytes, int m, int n, int k,
+                  int variant, int split_k, void* stream) {
+    int st = check_common(a, b, a_scale, b_scale, c, m, n, k);
+    if (st != FP8BS_OK) return st;
+    if (m == 0 || n == 0) return FP8BS_OK;
+    hipStream_t s = (hipStream_t)stream;
+    fp8bs_plan_t plan{};
+    if (k == 0) variant = FP8BS_VARIANT_GENERIC;   // empty sum: the generic kernel writes zeros
+    if (variant == FP8BS_VARIANT_AUTO) {
+        choose(m, n, k, 0, &plan);
+        if (split_k > 0) fill_plan(m, n, k, plan.variant, split_k, &plan);
+    } else {
+        VariantInfo vi{};
+        if (!variant_info(variant, &vi)) return FP8BS_ERR_BAD_VARIANT;
+        if (variant != FP8BS_VARIANT_GENERIC && ((m % 16) != 0 || (n % 16) != 0)) return FP8BS_ERR_BAD_VARIANT;
+        fill_plan(m, n, k, variant, split_k > 0 ? split_k : 1, &plan);
+    }
+    if (plan.split_k > 1 && (!ws || ws_bytes < plan.workspace_bytes)) return FP8BS_ERR_WORKSPACE;
+
+    fp8bs::GemmArgs g{};
+    g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.as = a_scale; g.bs = b_scale;
+    g.c = (uint16_t*)c; g.ws = (float*)ws; g.row_offsets = nullptr;
+    g.m = m; g.n = n; g.k = k; g.lda = m; g.nb = (n + 127) / 128;
+    g.split_k = plan.split_k;
+    g.kb_per_split = (int)cdiv(k / KBLK, plan.split_k);
+    g.band_h = 4;
+    g.num_experts = 0;
+    int mode = plan.split_k > 1 ? 1 : 0;
+    if (fp8bs::launch_gemm(plan.variant, mode, g, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
+    if (mode == 1) {
+        if (fp8bs::launch_splitk_reduce(g.ws, g.c, (size_t)m * n, plan.split_k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
+    }
+    return FP8BS_OK;
+}
+
+int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
+               void* c, void* ws, size_t ws_bytes, int m, int n, int k, void* stream) {
+    return fp8bs_gemm_ex(a, b, a_scale, b_scale, c, ws, ws_bytes, m, n, k, FP8BS_VARIANT_AUTO, 0, stream);
+}
+
+int fp8bs_gemm_grouped(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                       void* c, const int32_t* row_offsets, int num_experts, int total_rows,
+                       int n, int k, void* stream) {
+    if (num_experts <= 0) return FP8BS_ERR_BAD_OFFSETS;
+    if (!row_offsets) return FP8BS_ERR_NULL_POINTER;
+    int st = check_common(a, b, a_scale, b_scale, c, total_rows, n, k);
+    if (st != FP8BS_OK) return st;
+    if (total_rows == 0 || n == 0) return FP8BS_OK;
+    hipStream_t s = (hipStream_t)stream;
+    fp8bs::GemmArgs g{};
+    g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.as = a_scale; g.bs = b_scale;
+    g.c = (uint16_t*)c; g.ws = nullptr; g.row_offsets = row_offsets;
+    g.m = total_rows; g.n = n; g.k = k; g.lda = total_rows; g.nb = (n + 127) / 128;
+    g.split_k = 1; g.kb_per_split = k / KBLK; g.band_h = 4; g.num_experts = num_experts;
+    int variant = (k == 0 || (total_rows % 16) != 0 || (n % 16) != 0) ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
+    if (fp8bs::launch_gemm(variant, 2, g, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
+    return FP8BS_OK;
+}
+
+}  // extern "C"

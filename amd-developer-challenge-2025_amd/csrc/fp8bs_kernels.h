@@ -1,0 +1,32 @@
+// Internal interface between the C-ABI layer (fp8bs_api.hip) and the device code (fp8bs_kernels.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace fp8bs {
+
+// Kernel arguments. Layouts as in include/fp8bs.h. In grouped mode `m` and `lda` are the total row
+// count and `b`/`bs` carry a leading expert dimension.
+struct GemmArgs {
+    const uint8_t* a;
+    const uint8_t* b;
+    const float* as;
+    const float* bs;
+    uint16_t* c;            // bf16 bits
+    float* ws;              // split-K partial planes [split_k][m][n]
+    const int32_t* row_offsets;
+    int m, n, k;
+    int lda;                // bytes per k row of a (== m)
+    int nb;                 // ceil(n / 128)
+    int split_k, kb_per_split;
+    int band_h;             // tile rows per band of the tile walk
+    int num_experts;
+};
+
+// mode: 0 dense bf16, 1 dense split-K partials, 2 grouped.  variant: FP8BS_VARIANT_* (not AUTO).
+hipError_t launch_gemm(int variant, int mode, const GemmArgs& args, hipStream_t stream);
+hipError_t launch_splitk_reduce(const float* ws, uint16_t* c, size_t mn, int split_k, hipStream_t stream);
+int variant_lds_bytes(int variant);
+
+}  // namespace fp8bs

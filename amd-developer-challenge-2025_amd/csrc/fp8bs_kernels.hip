@@ -1,0 +1,482 @@
+// FP8 (OCP e4m3fn) block-scaled GEMM kernels for gfx950 (CDNA4, MI355X).
+//
+// Computes, per 128-wide K block kb,   P_kb[m][n] = sum_{kk in kb} A[m][kk] * B[n][kk]   on the FP8
+// matrix cores (v_mfma_f32_16x16x128_f8f6f4, one instruction = one whole scale block of one 16x16
+// tile), then folds   C[m][n] += P_kb[m][n] * (a_scale[m][kb] * b_scale[n/128][kb])   into fp32
+// accumulators on the vector ALU, and finally rounds to bf16.  Semantics follow the reference's
+// dequantise-then-multiply statement (1-amd-fp8-mm/0-amd-fp8-mm-new-begins.py:17-49, 85-89) and the
+// per-block fold of its shipped kernel (1-amd-fp8-mm/amd-fp8-mm-submission.py:333, 350-352).
+//
+// Memory layouts are the reference's (amd-fp8-mm-submission.py:66-75, 307-316): both operands arrive
+// with K as the strided dimension, a[kk*M + i], b[kk*N + j].  The K<->M/N transpose the matrix cores
+// need is fused into the LDS read: tiles are copied to LDS untransposed ([k][m] rows, 16-byte chunks,
+// asynchronous global->LDS loads that bypass registers) and the operands are fetched with the CDNA4
+// transposing read ds_read_b64_tr_b8, which hands every lane 8 consecutive-k bytes of one row.
+//
+// Layout facts used below were measured on the chip with one-hot operands:
+//  * ds_read_b64_tr_b8: inside each group of 16 lanes, source lanes 2r and 2r+1 address the low and
+//    high 8 bytes of "k row" r (r = 0..7); result lane i receives, as byte r, column i of row r.
+//  * v_mfma_f32_16x16x128_f8f6f4: lane l supplies 32 bytes of row l%16 for k group l/16; operand A
+//    and operand B use the same (group, byte) -> k map, so any k order inside the block is valid as
+//    long as both operands use the same one.  D[i][j] (i from src0 rows, j from src1 rows) lives in
+//    lane 16*(i/4) + j, register i%4.
+// The kernel feeds B rows (n) as src0 and A rows (m) as src1, so a lane owns four consecutive n of
+// one output row m: one a_scale value per lane per 16x16 tile and 8-byte contiguous bf16 stores.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include <type_traits>
+
+#include "fp8bs_kernels.h"
+
+namespace fp8bs {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef unsigned short v4us __attribute__((ext_vector_type(4)));
+
+#define LDS_V2I(p) ((__attribute__((address_space(3))) v2i*)(p))
+#define LDS_VOID(p) ((__attribute__((address_space(3))) void*)(p))
+
+static constexpr int KBLK = 128;  // scale block along K == K extent of one MFMA
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    v2f f = {lo, hi};
+    v2bf h = __builtin_convertvector(f, v2bf);   // v_cvt_pk_bf16_f32: round to nearest even
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+// 16 bytes per lane, global -> LDS without passing through registers (buffer_load_dwordx4 ... lds):
+// lane l's bytes land at lds_base + 16*l, lds_base must be wave-uniform; lanes whose offset is beyond
+// the buffer's size read zeros.
+__device__ __forceinline__ void copy16_global_to_lds(__amdgpu_buffer_rsrc_t rsrc, uint32_t lds_base, uint32_t byte_offset) {
+    asm volatile("s_mov_b32 m0, %2\n\tbuffer_load_dwordx4 %0, %1, 0 offen lds"
+                 :: "v"(byte_offset), "s"(rsrc), "s"(lds_base) : "memory", "m0");
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Tile -> workgroup mapping.  Workgroups are dealt round-robin to the 8 XCDs (each with its own L2),
+// so workgroup w lives on XCD w%8.  Give every XCD a contiguous run of "virtual" ids, and lay the
+// virtual ids over the tile grid in bands of GH tile rows walked column by column, so the tiles that
+// share an L2 form a compact block and re-use each other's A and B panels.
+// ---------------------------------------------------------------------------------------------------
+__device__ __forceinline__ int xcd_virtual_id(int wg, int total) {
+    const int NX = 8;
+    int x = wg % NX, idx = wg / NX;
+    int q = total / NX, r = total % NX;
+    return x * q + (x < r ? x : r) + idx;
+}
+
+__device__ __forceinline__ void band_tile(int v, int tiles_m, int tiles_n, int gh, int& tm, int& tn) {
+    int per_band = gh * tiles_n;
+    int band = v / per_band;
+    int rem = v - band * per_band;
+    int rows = tiles_m - band * gh;           // rows in this band (last band may be short)
+    rows = rows < gh ? rows : gh;
+    tn = rem / rows;
+    tm = band * gh + (rem - tn * rows);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Main kernel.
+//   BM x BN : workgroup tile (rows of A x rows of B), WM x WN : wave tile, 64*(BM/WM)*(BN/WN) threads.
+//   MODE 0  : dense, bf16 output
+//   MODE 1  : dense split-K, fp32 partial planes to the workspace
+//   MODE 2  : grouped (row_offsets), bf16 output
+// LDS: 2 stages, each [128 k][BM] bytes of A then [128 k][BN] bytes of B, 16-byte chunks XOR-swizzled
+// so that the 16 k rows touched by half a wave in one transposing read fall on 16 different 16-byte
+// bank groups.
+// ---------------------------------------------------------------------------------------------------
+template <int BM, int BN, int WM, int WN, int MODE>
+struct TileCfg {
+    static constexpr int WAVES_M = BM / WM, WAVES_N = BN / WN;
+    static constexpr int NWAVES = WAVES_M * WAVES_N;
+    static constexpr int NTHREADS = NWAVES * 64;
+    static constexpr int MT = WM / 16, NT = WN / 16;
+    static constexpr int CPR_A = BM / 16, CPR_B = BN / 16;          // 16-byte chunks per k row
+    static constexpr int A_BYTES = KBLK * BM, B_BYTES = KBLK * BN;
+    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+    static constexpr int A_LOADS = A_BYTES / 16 / NTHREADS;         // 16-byte loads per thread per block
+    static constexpr int B_LOADS = B_BYTES / 16 / NTHREADS;
+    static_assert(A_BYTES % (16 * NTHREADS) == 0 && B_BYTES % (16 * NTHREADS) == 0, "tile/threads");
+    static_assert(WN <= 128 && 128 % WN == 0, "a wave's n range must stay inside one b_scale block");
+    static_assert(CPR_A <= 16 && CPR_B <= 16, "swizzle assumes a k row spans at most 256 bytes");
+};
+
+template <int CPR>
+__device__ __forceinline__ int swz_of_krow(int krow) {
+    // rows per 256-byte bank sweep = 16/CPR; consecutive sweeps get consecutive XOR masks
+    return (krow / (16 / CPR)) % CPR;
+}
+
+template <int BM, int BN, int WM, int WN, int MODE>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64)
+void gemm_tr_kernel(const GemmArgs p) {
+    using C = TileCfg<BM, BN, WM, WN, MODE>;
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 4, i16 = lane & 15;
+    const int wave_m = wave % C::WAVES_M, wave_n = wave / C::WAVES_M;
+
+    // ---- which tile ---------------------------------------------------------------------------
+    int m0, n0, kb_begin, kb_end, split_z = 0;
+    int row_lo = 0, row_hi = p.m;                  // rows this workgroup may store
+    const uint8_t* bptr = p.b;
+    const float* bsptr = p.bs;
+    if (MODE == 2) {
+        // grouped: workgroup (blockIdx.x = tile_n, blockIdx.y = m-tile slot).  Slots are laid over
+        // the experts in order; expert e's tiles start at row_offsets[e] rounded down to 16 so that
+        // global 16-byte loads stay aligned; rows outside [row_offsets[e], row_offsets[e+1]) are
+        // computed but never stored.
+        int slot = blockIdx.y;
+        int e = 0, found = 0, start = 0, cnt_lo = 0, cnt_hi = 0;
+        int acc_tiles = 0;
+        for (int x = 0; x < p.num_experts; x++) {
+            int lo = p.row_offsets[x], hi = p.row_offsets[x + 1];
+            int s = lo & ~15;
+            int nt = (hi > lo) ? (hi - s + BM - 1) / BM : 0;
+            if (!found && slot < acc_tiles + nt) {
+                found = 1; e = x; start = s + (slot - acc_tiles) * BM; cnt_lo = lo; cnt_hi = hi;
+            }
+            acc_tiles += nt;
+        }
+        if (!found) return;                        // uniform for the whole workgroup
+        m0 = start; n0 = blockIdx.x * BN;
+        row_lo = cnt_lo; row_hi = cnt_hi;
+        bptr += (size_t)e * (size_t)p.k * (size_t)p.n;
+        bsptr += (size_t)e * (size_t)(p.k / KBLK) * (size_t)p.nb;
+        kb_begin = 0; kb_end = p.k / KBLK;
+    } else {
+        int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
+        int per_split = tiles_m * tiles_n;
+        int v = xcd_virtual_id(blockIdx.x, per_split * p.split_k);
+        split_z = v / per_split;
+        int tm, tn;
+        band_tile(v - split_z * per_split, tiles_m, tiles_n, p.band_h, tm, tn);
+        m0 = tm * BM; n0 = tn * BN;
+        int kbt = p.k / KBLK;
+        kb_begin = split_z * p.kb_per_split;
+        kb_end = kb_begin + p.kb_per_split;
+        kb_end = kb_end < kbt ? kb_end : kbt;
+    }
+
+    // ---- buffer resources: out-of-range lanes read zeros instead of faulting -------------------
+    const uint32_t a_bytes = (uint32_t)p.k * (uint32_t)p.lda;
+    const uint32_t b_bytes = (uint32_t)p.k * (uint32_t)p.n;
+    __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, a_bytes, 0x00020000);
+    __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)bptr, 0, b_bytes, 0x00020000);
+
+    // ---- global -> LDS copy plan: wave w, instruction i fills 1 KiB of LDS starting at chunk slot
+    //      (i*NWAVES + w)*64; lane l fills slot P = that + l.  Slot P holds k row P/CPR, stored chunk
+    //      P%CPR, which is logical chunk (P%CPR) ^ swz(k row): pick the global address accordingly.
+    uint32_t a_goff[C::A_LOADS], b_goff[C::B_LOADS];
+#pragma unroll
+    for (int i = 0; i < C::A_LOADS; i++) {
+        int P = (i * C::NWAVES + wave) * 64 + lane;
+        int krow = P / C::CPR_A, cs = P % C::CPR_A;
+        int c = cs ^ swz_of_krow<C::CPR_A>(krow);
+        a_goff[i] = (uint32_t)(kb_begin * KBLK + krow) * (uint32_t)p.lda + (uint32_t)(m0 + 16 * c);
+    }
+#pragma unroll
+    for (int i = 0; i < C::B_LOADS; i++) {
+        int P = (i * C::NWAVES + wave) * 64 + lane;
+        int krow = P / C::CPR_B, cs = P % C::CPR_B;
+        int c = cs ^ swz_of_krow<C::CPR_B>(krow);
+        b_goff[i] = (uint32_t)(kb_begin * KBLK + krow) * (uint32_t)p.n + (uint32_t)(n0 + 16 * c);
+    }
+    const uint32_t a_kstep = (uint32_t)KBLK * (uint32_t)p.lda, b_kstep = (uint32_t)KBLK * (uint32_t)p.n;
+
+    // The copies are issued from inline assembly so that the compiler's hazard tracking does not see
+    // them: it cannot tell that a copy into one stage never aliases the transposing reads of the other
+    // stage and would otherwise make every LDS read wait for all outstanding copies.  Completion is
+    // enforced by hand: s_waitcnt vmcnt(0) + workgroup barrier before the first read of a stage.
+    const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    auto issue_loads = [&](int stage) {
+        const uint32_t sa = lds_base + stage * C::STAGE_BYTES + wave * 1024;
+        const uint32_t sb = sa + C::A_BYTES;
+#pragma unroll
+        for (int i = 0; i < C::A_LOADS; i++) {
+            copy16_global_to_lds(a_rsrc, sa + i * C::NWAVES * 1024, a_goff[i]);
+            a_goff[i] += a_kstep;
+        }
+#pragma unroll
+        for (int i = 0; i < C::B_LOADS; i++) {
+            copy16_global_to_lds(b_rsrc, sb + i * C::NWAVES * 1024, b_goff[i]);
+            b_goff[i] += b_kstep;
+        }
+    };
+
+    // ---- per-lane LDS read addresses -----------------------------------------------------------
+    // transposing read j of a 16-row tile: k rows 32j + 8g + (i16>>1), byte half (i16&1)
+    const int krow_lane = 8 * g + (i16 >> 1);
+    const int swz_a = swz_of_krow<C::CPR_A>(krow_lane);     // independent of j (32j is a multiple of 16)
+    const int swz_b = swz_of_krow<C::CPR_B>(krow_lane);
+    const int a_lane_off = krow_lane * BM + (i16 & 1) * 8;
+    const int b_lane_off = C::A_BYTES + krow_lane * BN + (i16 & 1) * 8;
+    const int a_chunk0 = wave_m * (WM / 16), b_chunk0 = wave_n * (WN / 16);
+
+    auto read_a = [&](v8i& dst, int t, const unsigned char* sbase) {
+        const unsigned char* q = sbase + a_lane_off + (((a_chunk0 + t) ^ swz_a) << 4);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v2i x = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_V2I(q + j * 32 * BM));
+            dst[2 * j] = x[0]; dst[2 * j + 1] = x[1];
+        }
+    };
+    auto read_b = [&](v8i& dst, int u, const unsigned char* sbase) {
+        const unsigned char* q = sbase + b_lane_off + (((b_chunk0 + u) ^ swz_b) << 4);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v2i x = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_V2I(q + j * 32 * BN));
+            dst[2 * j] = x[0]; dst[2 * j + 1] = x[1];
+        }
+    };
+
+    // ---- scales -------------------------------------------------------------------------------
+    // lane's output row for m-tile t is  m0 + wave_m*WM + 16t + i16 ; clamp so tail lanes stay in range
+    uint32_t as_off[C::MT];
+#pragma unroll
+    for (int t = 0; t < C::MT; t++) {
+        int r = m0 + wave_m * WM + 16 * t + i16;
+        r = r < p.lda - 1 ? r : p.lda - 1;
+        as_off[t] = (uint32_t)r;
+    }
+    int nblk = (n0 + wave_n * WN) / 128;
+    nblk = __builtin_amdgcn_readfirstlane(nblk < p.nb - 1 ? nblk : p.nb - 1);
+
+    v4f acc[C::MT][C::NT];
+#pragma unroll
+    for (int t = 0; t < C::MT; t++)
+#pragma unroll
+        for (int u = 0; u < C::NT; u++) acc[t][u] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    const int nkb = kb_end - kb_begin;
+    if (nkb > 0) {
+        // ---- prologue: block 0 -> stage 0, wait, then block 1 -> stage 1 in the background ----
+        const float* as_row = p.as + (size_t)kb_begin * p.lda;     // a_scale row of the current k block
+        const float* bs_row = bsptr + (size_t)kb_begin * p.nb;
+        float as_cur[C::MT], bs_cur;
+        issue_loads(0);
+#pragma unroll
+        for (int t = 0; t < C::MT; t++) as_cur[t] = as_row[as_off[t]];
+        bs_cur = bs_row[nblk];
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+        __syncthreads();
+        if (nkb > 1) issue_loads(1);
+
+        v8i areg[C::MT], breg[2];
+#pragma unroll
+        for (int t = 0; t < C::MT; t++) read_a(areg[t], t, lds);
+        read_b(breg[0], 0, lds);
+
+        constexpr int STEPS = C::MT * C::NT;
+        constexpr int LAG = 3, RING = 4;      // fold the result of step s-LAG while step s runs
+
+        // One K block.  HAS_NEXT is a compile-time flag so that the step sequence below is a single
+        // straight-line block for the instruction scheduler.
+        auto k_block = [&](const unsigned char* sbase, const unsigned char* snext, auto has_next_tag) {
+            constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
+            float sc[C::MT];
+#pragma unroll
+            for (int t = 0; t < C::MT; t++) sc[t] = as_cur[t] * bs_cur;
+            if (HAS_NEXT) {
+                as_row += p.lda; bs_row += p.nb;
+#pragma unroll
+                for (int t = 0; t < C::MT; t++) as_cur[t] = as_row[as_off[t]];
+                bs_cur = bs_row[nblk];
+            }
+            v4f ring[RING];
+#pragma unroll
+            for (int s = 0; s < STEPS + LAG; s++) {
+                if (s < STEPS) {
+                    const int u = s / C::MT, t = s % C::MT;
+                    if (t == 0 && u + 1 < C::NT) read_b(breg[(u + 1) & 1], u + 1, sbase);
+                    if (t == 0 && u == C::NT - 1) {
+                        // All reads of this stage are issued.  Wait for them and for this wave's part
+                        // of the next block, then meet the other waves: after the barrier the next
+                        // block is complete in the other stage and this stage may be overwritten.
+                        __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
+                        __syncthreads();
+                    }
+                    const v4f z = {0.f, 0.f, 0.f, 0.f};
+                    ring[s % RING] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(breg[u & 1], areg[t], z, 0, 0, 0, 0, 0, 0);
+                    if (u == C::NT - 1 && HAS_NEXT) {
+                        // operands of the next block, fetched while the last MFMAs of this one run
+                        read_a(areg[t], t, snext);
+                        if (t == 0) read_b(breg[0], 0, snext);
+                    }
+                }
+                if (s >= LAG) {
+                    const int sp = s - LAG, u = sp / C::MT, t = sp % C::MT;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc[t][u][r] = __builtin_fmaf(ring[sp % RING][r], sc[t], acc[t][u][r]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+
+        int i = 0;
+        for (; i + 1 < nkb; i++) {
+            k_block(lds + (i & 1) * C::STAGE_BYTES, lds + ((i & 1) ^ 1) * C::STAGE_BYTES, std::true_type{});
+            // Block i+2 goes into the stage just released.  Issued unconditionally to keep the loop
+            // a single basic block: past the end of K the buffer bounds make the copy read zeros (or,
+            // for a K split, the next split's bytes) into a stage nobody reads again, and the final
+            // block below waits for all copies before the workgroup ends.
+            issue_loads(i & 1);
+        }
+        k_block(lds + (i & 1) * C::STAGE_BYTES, lds, std::false_type{});
+    }
+
+    // ---- epilogue -----------------------------------------------------------------------------
+#pragma unroll
+    for (int t = 0; t < C::MT; t++) {
+        const int row = m0 + wave_m * WM + 16 * t + i16;
+        if (row < row_lo || row >= row_hi) continue;
+#pragma unroll
+        for (int u = 0; u < C::NT; u++) {
+            const int col = n0 + wave_n * WN + 16 * u + 4 * g;
+            if (col >= p.n) continue;
+            if (MODE == 1) {
+                float* dst = p.ws + ((size_t)split_z * p.m + row) * (size_t)p.n + col;
+                *(v4f*)dst = acc[t][u];
+            } else {
+                v2i o;
+                o[0] = (int)pack_bf16x2(acc[t][u][0], acc[t][u][1]);
+                o[1] = (int)pack_bf16x2(acc[t][u][2], acc[t][u][3]);
+                *(v2i*)(p.c + (size_t)row * p.n + col) = o;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Split-K reduction: sums `split_k` fp32 planes in a fixed order and rounds to bf16, 8 outputs per
+// thread with one 16-byte store (role of fp8_mm_128x128_ft2_split4_merge,
+// 1-amd-fp8-mm/amd-fp8-mm-submission.py:485-511, for any split count).
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256)
+void splitk_reduce_kernel(const float* __restrict__ ws, uint16_t* __restrict__ c, size_t mn, int split_k) {
+    size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (i >= mn) return;
+    v4f s0 = *(const v4f*)(ws + i), s1 = *(const v4f*)(ws + i + 4);
+    for (int z = 1; z < split_k; z++) {
+        s0 += *(const v4f*)(ws + (size_t)z * mn + i);
+        s1 += *(const v4f*)(ws + (size_t)z * mn + i + 4);
+    }
+    v4i o;
+    o[0] = (int)pack_bf16x2(s0[0], s0[1]); o[1] = (int)pack_bf16x2(s0[2], s0[3]);
+    o[2] = (int)pack_bf16x2(s1[0], s1[1]); o[3] = (int)pack_bf16x2(s1[2], s1[3]);
+    *(v4i*)(c + i) = o;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Generic kernel: any m, n (no alignment requirement), one output element per thread, scalar decode.
+// Only used when m or n is not a multiple of 16, where the 16-byte tile copies above cannot be used.
+// Also handles the grouped case (row_offsets != nullptr).
+// ---------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float e4m3fn_to_float(uint32_t v) {
+    uint32_t s = (v & 0x80u) << 24, e = (v >> 3) & 15u, m = v & 7u;
+    float f;
+    if (e == 0) f = (float)m * 0.001953125f;                         // subnormal: m * 2^-9
+    else if (e == 15 && m == 7) f = __builtin_nanf("");
+    else f = __builtin_bit_cast(float, ((e + 120u) << 23) | (m << 20));
+    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, f) | s);
+}
+
+__global__ __launch_bounds__(256)
+void gemm_generic_kernel(const GemmArgs p) {
+    int col = blockIdx.x * 16 + (threadIdx.x & 15);
+    int row = blockIdx.y * 16 + (threadIdx.x >> 4);
+    if (row >= p.m || col >= p.n) return;
+    const uint8_t* b = p.b;
+    const float* bs = p.bs;
+    if (p.row_offsets) {
+        int e = 0;
+        while (e + 1 < p.num_experts && row >= p.row_offsets[e + 1]) e++;
+        b += (size_t)e * p.k * p.n;
+        bs += (size_t)e * (p.k / KBLK) * p.nb;
+    }
+    float accum = 0.f;
+    for (int kb = 0; kb < p.k / KBLK; kb++) {
+        float part = 0.f;
+        for (int kk = kb * KBLK; kk < (kb + 1) * KBLK; kk++)
+            part = __builtin_fmaf(e4m3fn_to_float(p.a[(size_t)kk * p.lda + row]), e4m3fn_to_float(b[(size_t)kk * p.n + col]), part);
+        accum = __builtin_fmaf(part, p.as[(size_t)kb * p.lda + row] * bs[(size_t)kb * p.nb + col / 128], accum);
+    }
+    v2f f = {accum, 0.f};
+    v2bf h = __builtin_convertvector(f, v2bf);
+    p.c[(size_t)row * p.n + col] = __builtin_bit_cast(uint32_t, h) & 0xFFFFu;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Launchers
+// ---------------------------------------------------------------------------------------------------
+template <int BM, int BN, int WM, int WN, int MODE>
+static hipError_t launch_tr(const GemmArgs& a, dim3 grid, hipStream_t stream) {
+    using C = TileCfg<BM, BN, WM, WN, MODE>;
+    auto kern = gemm_tr_kernel<BM, BN, WM, WN, MODE>;
+    static bool attr_done = false;   // raising the dynamic-LDS limit is idempotent; a race is harmless
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
+    return hipGetLastError();
+}
+
+template <int BM, int BN, int WM, int WN>
+static hipError_t launch_shape(const GemmArgs& a, int mode, hipStream_t stream) {
+    if (mode == 2) {
+        int tiles_n = (a.n + BN - 1) / BN;
+        // upper bound on m-tile slots: every expert can waste up to 15 rows (aligned-down start)
+        // plus one partial tile
+        long slots = ((long)a.m + BM - 1) / BM + 2L * a.num_experts;
+        return launch_tr<BM, BN, WM, WN, 2>(a, dim3(tiles_n, (unsigned)slots), stream);
+    }
+    int tiles = ((a.m + BM - 1) / BM) * ((a.n + BN - 1) / BN) * a.split_k;
+    if (mode == 1) return launch_tr<BM, BN, WM, WN, 1>(a, dim3(tiles), stream);
+    return launch_tr<BM, BN, WM, WN, 0>(a, dim3(tiles), stream);
+}
+
+hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t stream) {
+    switch (variant) {
+        case 1: {
+            dim3 grid((a.n + 15) / 16, (a.m + 15) / 16);
+            hipLaunchKernelGGL(gemm_generic_kernel, grid, dim3(256), 0, stream, a);
+            return hipGetLastError();
+        }
+        case 2: return launch_shape<256, 256, 64, 128>(a, mode, stream);
+        case 3: return launch_shape<128, 128, 64, 64>(a, mode, stream);
+        case 4: return launch_shape<64, 128, 32, 64>(a, mode, stream);
+        case 5: return launch_shape<256, 128, 64, 64>(a, mode, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_splitk_reduce(const float* ws, uint16_t* c, size_t mn, int split_k, hipStream_t stream) {
+    size_t threads = (mn + 7) / 8;
+    unsigned blocks = (unsigned)((threads + 255) / 256);
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, stream, ws, c, mn, split_k);
+    return hipGetLastError();
+}
+
+int variant_lds_bytes(int variant) {
+    switch (variant) {
+        case 2: return TileCfg<256, 256, 64, 128, 0>::LDS_BYTES;
+        case 3: return TileCfg<128, 128, 64, 64, 0>::LDS_BYTES;
+        case 4: return TileCfg<64, 128, 32, 64, 0>::LDS_BYTES;
+        case 5: return TileCfg<256, 128, 64, 64, 0>::LDS_BYTES;
+        default: return 0;
+    }
+}
+
+}  // namespace fp8bs

@@ -1,0 +1,110 @@
+/*
+ * fp8bs.h - C ABI of libfp8bs.so: FP8 (OCP e4m3fn) block-scaled GEMM for gfx950 (MI355X).
+ *
+ *   C[m][n] (bf16) = sum_kb ( sum_{kk in block kb} A[m][kk] * B[n][kk] ) * a_scale[m][kb] * b_scale[n/128][kb]
+ *
+ * This header is the drop-in boundary for the host launcher of the reference
+ * (1-amd-fp8-mm/amd-fp8-mm-submission.py:8 and :514-579, `void fp8_mm(torch::Tensor a, b, as, bs,
+ * c, c_tmp)`), re-cut as plain pointers and sizes so that any host language can bind it.
+ *
+ * Physical layouts (the reference's, 1-amd-fp8-mm/amd-fp8-mm-submission.py:66-75, 307-316, 364):
+ *   a        : K rows of M bytes       a[kk * M + i]                 e4m3fn
+ *   b        : K rows of N bytes       b[kk * N + j]                 e4m3fn
+ *   a_scale  : K/128 rows of M floats  a_scale[(kk/128) * M + i]
+ *   b_scale  : K/128 rows of NB floats b_scale[(kk/128) * NB + j/128],  NB = ceil(N/128)
+ *   c        : M rows of N bf16        c[i * N + j]
+ * All pointers are device pointers. The library never allocates or frees device memory and writes
+ * nothing but `c` and the caller's workspace `ws`. Calls are asynchronous on `stream`
+ * (a hipStream_t passed as void*; NULL = the null stream). K must be a multiple of 128.
+ */
+#ifndef FP8BS_H
+#define FP8BS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes (0 = success). The reference launcher returns void and never reads launch errors
+ * (1-amd-fp8-mm/amd-fp8-mm-submission.py:514-579); this boundary reports them. */
+enum {
+    FP8BS_OK = 0,
+    FP8BS_ERR_NULL_POINTER = 1,   /* a required pointer is NULL                             */
+    FP8BS_ERR_BAD_SHAPE = 2,      /* m,n,k <= 0 where not allowed, or k % 128 != 0           */
+    FP8BS_ERR_WORKSPACE = 3,      /* ws is NULL / smaller than fp8bs_workspace_bytes(...)    */
+    FP8BS_ERR_TOO_LARGE = 4,      /* an operand exceeds the 4 GiB buffer-addressing limit    */
+    FP8BS_ERR_LAUNCH = 5,         /* hipGetLastError() after launch was not hipSuccess       */
+    FP8BS_ERR_BAD_OFFSETS = 6,    /* grouped: bad expert count                               */
+    FP8BS_ERR_BAD_VARIANT = 7     /* forced variant id unknown or not applicable             */
+};
+
+/* Kernel variants the planner chooses from. */
+enum {
+    FP8BS_VARIANT_AUTO = 0,
+    FP8BS_VARIANT_GENERIC = 1,    /* scalar kernel, any m/n (alignment fallback)             */
+    FP8BS_VARIANT_T256x256 = 2,   /* compute-bound: 256x256 tile, 8 waves                    */
+    FP8BS_VARIANT_T128x128 = 3,   /* mid-size: 128x128 tile, 4 waves                         */
+    FP8BS_VARIANT_T64x128 = 4,    /* skinny-M: 64(m) x 128(n) tile, 4 waves, split-K         */
+    FP8BS_VARIANT_T256x128 = 5,   /* 256(m) x 128(n) tile, 8 waves                           */
+    FP8BS_VARIANT_COUNT = 6
+};
+
+/* What fp8bs_plan() decides for a shape. Replaces the exact-(m,n,k) if-ladder of the reference
+ * (1-amd-fp8-mm/amd-fp8-mm-submission.py:528-578) with a shape-family rule. */
+typedef struct fp8bs_plan_t {
+    int32_t variant;        /* FP8BS_VARIANT_*                                   */
+    int32_t tile_m, tile_n; /* workgroup tile                                    */
+    int32_t split_k;        /* number of K partitions (1 = no workspace needed)  */
+    int32_t grid_x, grid_y, grid_z;
+    int32_t block_threads;
+    int32_t lds_bytes;
+    int32_t reserved;
+    uint64_t workspace_bytes;
+} fp8bs_plan_t;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int fp8bs_version(void);
+
+/* Human-readable text of a status code. Never NULL. */
+const char* fp8bs_strerror(int status);
+
+/* Host-only planning: no GPU needed. Replaces the dispatch of
+ * 1-amd-fp8-mm/amd-fp8-mm-submission.py:528-578. `num_cus` <= 0 means 256 (MI355X). */
+int fp8bs_plan(int m, int n, int k, int num_cus, fp8bs_plan_t* out);
+
+/* Bytes of device workspace fp8bs_gemm needs for this shape (0 when split_k == 1). Replaces the
+ * per-call `torch.empty(m*n*4)` of 1-amd-fp8-mm/amd-fp8-mm-submission.py:600: the caller owns and
+ * reuses the workspace. */
+size_t fp8bs_workspace_bytes(int m, int n, int k);
+
+/* Dense GEMM. Replaces `fp8_mm(a,b,as,bs,c,c_tmp)`,
+ * 1-amd-fp8-mm/amd-fp8-mm-submission.py:514-579. Inputs are never modified (the reference's
+ * pre-transpose branch, :570-571, overwrites a and b; this one does not). */
+int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
+               void* c, void* ws, size_t ws_bytes, int m, int n, int k, void* stream);
+
+/* Same as fp8bs_gemm with the variant and split-K forced (testing and benchmarking the shape
+ * families against each other). variant = FP8BS_VARIANT_AUTO and split_k = 0 reproduce fp8bs_gemm.
+ * Workspace requirement for a forced split_k > 1: split_k * m * n * 4 bytes. */
+int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                  void* c, void* ws, size_t ws_bytes, int m, int n, int k,
+                  int variant, int split_k, void* stream);
+
+/* Grouped (MoE expert) GEMM. Row-offset convention of 2-amd-moe/3-amd-fp8-moe-hip-myhgemm.py:142-148
+ * and :328-336 (expert_offset = exclusive prefix sum of per-expert row counts), with the total
+ * appended: row_offsets has num_experts+1 int32 entries on the device, row_offsets[0] = 0,
+ * row_offsets[num_experts] = total_rows. Expert e owns rows [row_offsets[e], row_offsets[e+1]).
+ *   a        : K rows of total_rows bytes (permuted, expert-contiguous rows), a_scale likewise
+ *   b        : num_experts matrices, each K rows of N bytes;  b_scale: num_experts x (K/128) x NB
+ *   c        : total_rows rows of N bf16
+ * No host synchronisation (the reference needs one to size its grid, :595, :607-610). */
+int fp8bs_gemm_grouped(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                       void* c, const int32_t* row_offsets, int num_experts, int total_rows,
+                       int n, int k, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FP8BS_H */
