@@ -1,0 +1,15 @@
+"""MI355X-native FP8 block-scaled GEMM behind the reference's ``custom_kernel(data)`` entry point.
+
+The directory name is not a Python identifier; import it with
+``importlib.import_module("amd-developer-challenge-2025_amd")`` (the repository root's ``submission.py``
+does exactly that and re-exports ``custom_kernel``).
+
+Layout of the package:
+  csrc/           hand-written HIP kernels (gfx950) and the C ABI (include/fp8bs.h)
+  build.py        compiles csrc/ into libfp8bs.so next to this file
+  _lib.py         ctypes binding of the C ABI; raises if the library is missing
+  submission.py   custom_kernel(data) / grouped_kernel(data): the reference's Python entry points
+  inputs.py       e4m3fn block quantisers and the synthetic inputs of the benchmark configurations
+"""
+from .submission import custom_kernel, grouped_kernel, plan, workspace_bytes  # noqa: F401
+from . import inputs  # noqa: F401

@@ -1,0 +1,66 @@
+"""ctypes binding of libfp8bs.so (C ABI declared in include/fp8bs.h).
+
+There is no fallback: if the library has not been built the import of the entry points fails
+loudly, so a GPU run can never silently take another path.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libfp8bs.so")
+
+# Every symbol include/fp8bs.h declares.
+EXPORTS = (
+    "fp8bs_version", "fp8bs_strerror", "fp8bs_plan", "fp8bs_workspace_bytes",
+    "fp8bs_gemm", "fp8bs_gemm_ex", "fp8bs_gemm_grouped",
+)
+
+VARIANT_NAMES = {0: "auto", 1: "generic", 2: "t256x256", 3: "t128x128", 4: "t64x128", 5: "t256x128"}
+
+
+class Plan(ctypes.Structure):
+    """Mirror of fp8bs_plan_t."""
+    _fields_ = [
+        ("variant", ctypes.c_int32), ("tile_m", ctypes.c_int32), ("tile_n", ctypes.c_int32),
+        ("split_k", ctypes.c_int32), ("grid_x", ctypes.c_int32), ("grid_y", ctypes.c_int32),
+        ("grid_z", ctypes.c_int32), ("block_threads", ctypes.c_int32), ("lds_bytes", ctypes.c_int32),
+        ("reserved", ctypes.c_int32), ("workspace_bytes", ctypes.c_uint64),
+    ]
+
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the library once; raise RuntimeError if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "libfp8bs.so is not built (%s missing): run `python __graft_entry__.py` or "
+            "`python amd-developer-challenge-2025_amd/build.py`; there is no fallback path" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, i32, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    lib.fp8bs_version.restype = i32
+    lib.fp8bs_version.argtypes = []
+    lib.fp8bs_strerror.restype = ctypes.c_char_p
+    lib.fp8bs_strerror.argtypes = [i32]
+    lib.fp8bs_plan.restype = i32
+    lib.fp8bs_plan.argtypes = [i32, i32, i32, i32, ctypes.POINTER(Plan)]
+    lib.fp8bs_workspace_bytes.restype = sz
+    lib.fp8bs_workspace_bytes.argtypes = [i32, i32, i32]
+    lib.fp8bs_gemm.restype = i32
+    lib.fp8bs_gemm.argtypes = [vp, vp, vp, vp, vp, vp, sz, i32, i32, i32, vp]
+    lib.fp8bs_gemm_ex.restype = i32
+    lib.fp8bs_gemm_ex.argtypes = [vp, vp, vp, vp, vp, vp, sz, i32, i32, i32, i32, i32, vp]
+    lib.fp8bs_gemm_grouped.restype = i32
+    lib.fp8bs_gemm_grouped.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]
+    _lib = lib
+    return lib
+
+
+def check(status: int) -> None:
+    """Raise RuntimeError with the library's message for a non-zero status."""
+    if status != 0:
+        raise RuntimeError("fp8bs: %s (status %d)" % (load().fp8bs_strerror(status).decode(), status))

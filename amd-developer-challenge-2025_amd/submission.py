@@ -1,0 +1,132 @@
+"""``custom_kernel(data)``: the reference's Python entry point, backed by libfp8bs.so.
+
+Mirrors 1-amd-fp8-mm/amd-fp8-mm-submission.py:594-604 (contract docstring:
+1-amd-fp8-mm/0-amd-fp8-mm-new-begins.py:66-77): ``data = (a, b, a_scale, b_scale, c)``, ``c`` is
+filled in place and the same tensor object is returned.  Tensors arrive in the reference's layouts:
+
+    a        [m, k]          float8_e4m3fn   stride (1, m)      (K-major: storage is [k][m])
+    b        [n, k]          float8_e4m3fn   stride (1, n)
+    a_scale  [m, k/128]      float32         stride (1, m)
+    b_scale  [ceil(n/128), k/128] float32    stride (1, ceil(n/128))
+    c        [m, n]          bfloat16        contiguous
+
+Differences from the reference, by design: OCP e4m3fn instead of e4m3fnuz (gfx950's FP8), the launch
+goes to torch's current stream instead of the null stream, errors raise instead of being dropped,
+the split-K workspace is cached per device instead of allocated per call
+(amd-fp8-mm-submission.py:600), and ``a``/``b`` are never written (the reference's pre-transpose
+branch overwrites them, :570-571).
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+_workspaces = {}   # device index -> uint8 tensor, grown on demand, reused across calls
+
+
+def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    ws = _workspaces.get(device.index)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[device.index] = ws
+    return ws
+
+
+def _is_kmajor(t: torch.Tensor) -> bool:
+    """True if the 2-D tensor's storage is its transpose laid out contiguously (stride (1, rows))."""
+    return t.dim() == 2 and t.t().is_contiguous()
+
+
+def _check_operands(a, b, a_scale, b_scale, c, rows, n, k):
+    if a.dtype != torch.float8_e4m3fn or b.dtype != torch.float8_e4m3fn:
+        raise TypeError("a and b must be torch.float8_e4m3fn")
+    if a_scale.dtype != torch.float32 or b_scale.dtype != torch.float32:
+        raise TypeError("a_scale and b_scale must be torch.float32")
+    if c.dtype != torch.bfloat16:
+        raise TypeError("c must be torch.bfloat16")
+    if k % 128 != 0:
+        raise ValueError("k must be a multiple of 128 (got %d)" % k)
+    for name, t in (("a", a), ("b", b), ("a_scale", a_scale), ("b_scale", b_scale), ("c", c)):
+        if not t.is_cuda:
+            raise ValueError("%s must be a GPU tensor: this path has no CPU implementation" % name)
+        if t.device != a.device:
+            raise ValueError("all tensors must be on the same device")
+    if a.shape[1] != k or tuple(a_scale.shape) != (rows, k // 128):
+        raise ValueError("a / a_scale shapes do not match [rows, k] / [rows, k/128]")
+    if not _is_kmajor(a) or not _is_kmajor(a_scale):
+        raise ValueError("a and a_scale must be K-major (stride (1, rows)), as the reference lays them out")
+    if not c.is_contiguous() or tuple(c.shape) != (rows, n):
+        raise ValueError("c must be a contiguous [rows, n] tensor")
+
+
+def plan(m: int, n: int, k: int) -> _lib.Plan:
+    """The kernel variant, split-K and grid the library would choose for a dense shape (host only)."""
+    p = _lib.Plan()
+    _lib.check(_lib.load().fp8bs_plan(m, n, k, 0, ctypes.byref(p)))
+    return p
+
+
+def workspace_bytes(m: int, n: int, k: int) -> int:
+    return int(_lib.load().fp8bs_workspace_bytes(m, n, k))
+
+
+def custom_kernel(data, variant: int = 0, split_k: int = 0):
+    """Block-scale fp8 gemm: fills and returns ``c`` (see module docstring for the layouts).
+
+    ``variant``/``split_k`` force a kernel variant (FP8BS_VARIANT_*) and a K split for testing;
+    the defaults let the library's planner decide.
+    """
+    a, b, a_scale, b_scale, c = data
+    m, k = a.shape
+    n = b.shape[0]
+    _check_operands(a, b, a_scale, b_scale, c, m, n, k)
+    nb = (n + 127) // 128
+    if b.shape[1] != k or tuple(b_scale.shape) != (nb, k // 128):
+        raise ValueError("b / b_scale shapes do not match [n, k] / [ceil(n/128), k/128]")
+    if not _is_kmajor(b) or not _is_kmajor(b_scale):
+        raise ValueError("b and b_scale must be K-major (stride (1, n) / (1, ceil(n/128)))")
+    lib = _lib.load()
+    if variant == 0 and split_k == 0:
+        need = workspace_bytes(m, n, k) if (m > 0 and n > 0 and k > 0) else 0
+    else:
+        need = max(split_k, 1) * m * n * 4 if split_k > 1 else 0
+    ws_ptr, ws_len = None, 0
+    if need:
+        ws = _workspace(a.device, need)
+        ws_ptr, ws_len = ws.data_ptr(), ws.numel()
+    with torch.cuda.device(a.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        st = lib.fp8bs_gemm_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
+                               c.data_ptr(), ws_ptr, ws_len, m, n, k, variant, split_k, stream)
+    _lib.check(st)
+    return c
+
+
+def grouped_kernel(data):
+    """Grouped (MoE expert) variant: ``data = (a, b, a_scale, b_scale, row_offsets, c)``.
+
+    Row-offset convention of 2-amd-moe/3-amd-fp8-moe-hip-myhgemm.py:142-148, :328-336 with the
+    total appended: ``row_offsets`` is int32 [E+1] on the GPU, expert e owns rows
+    [row_offsets[e], row_offsets[e+1]) of the expert-contiguous ``a`` ([rows, k], K-major) and ``c``
+    ([rows, n]).  ``b`` is [E, n, k] with each expert K-major (stride (n*k, 1, n)); ``b_scale`` is
+    [E, ceil(n/128), k/128] with stride (nb*kb, 1, nb).  Fills and returns ``c``; no host sync.
+    """
+    a, b, a_scale, b_scale, row_offsets, c = data
+    rows, k = a.shape
+    num_experts, n = b.shape[0], b.shape[1]
+    _check_operands(a, b, a_scale, b_scale, c, rows, n, k)
+    nb, kb = (n + 127) // 128, k // 128
+    if tuple(b.shape) != (num_experts, n, k) or tuple(b_scale.shape) != (num_experts, nb, kb):
+        raise ValueError("b / b_scale shapes do not match [E, n, k] / [E, ceil(n/128), k/128]")
+    if not b.transpose(1, 2).is_contiguous() or not b_scale.transpose(1, 2).is_contiguous():
+        raise ValueError("every expert of b and b_scale must be K-major")
+    if row_offsets.dtype != torch.int32 or tuple(row_offsets.shape) != (num_experts + 1,) or not row_offsets.is_cuda:
+        raise ValueError("row_offsets must be an int32 GPU tensor with num_experts+1 entries")
+    lib = _lib.load()
+    with torch.cuda.device(a.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        st = lib.fp8bs_gemm_grouped(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
+                                    c.data_ptr(), row_offsets.data_ptr(), num_experts, rows, n, k, stream)
+    _lib.check(st)
+    return c

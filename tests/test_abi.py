@@ -1,0 +1,81 @@
+"""The C-ABI library loads without a GPU, exports every symbol include/fp8bs.h declares, and its
+host-only entry points (planner, argument checks, error strings) behave.  No GPU compute here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from conftest import ROOT
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "fp8bs.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fp8bs_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    lib = pkg._lib.load()
+    declared = _declared_symbols()
+    assert set(declared) == set(pkg._lib.EXPORTS)
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.fp8bs_version() >= 100
+
+
+def test_plan_shape_families(pkg):
+    p = pkg.plan(4096, 4096, 4096)
+    assert p.variant == 2 and (p.tile_m, p.tile_n) == (256, 256) and p.split_k == 1 and p.workspace_bytes == 0
+    assert p.grid_x == 256 and p.block_threads == 512 and p.lds_bytes == 131072
+    p = pkg.plan(64, 18432, 7168)                       # skinny-M: small tile, split-K, workspace
+    assert p.variant == 4 and p.tile_m == 64 and p.split_k > 1
+    assert p.workspace_bytes == p.split_k * 64 * 18432 * 4 == pkg.workspace_bytes(64, 18432, 7168)
+    p = pkg.plan(130, 192, 256)                         # not a multiple of 16 -> generic kernel
+    assert p.variant == 1 and p.split_k == 1
+    p = pkg.plan(256, 512, 1024)
+    assert p.variant in (3, 5) and p.split_k >= 1 and p.split_k <= 8
+
+
+def test_plan_rejects_bad_shapes(pkg):
+    lib = pkg._lib.load()
+    out = pkg._lib.Plan()
+    assert lib.fp8bs_plan(16, 16, 100, 0, ctypes.byref(out)) == 2      # k not a multiple of 128
+    assert lib.fp8bs_plan(0, 16, 128, 0, ctypes.byref(out)) == 2
+    assert lib.fp8bs_plan(16, 16, 128, 0, None) == 1
+    assert pkg.workspace_bytes(16, 16, 100) == 0
+
+
+def test_argument_errors_are_reported_before_any_launch(pkg):
+    lib = pkg._lib.load()
+    one = ctypes.c_void_p(16)      # never dereferenced: the checks fail first
+    assert lib.fp8bs_gemm(one, one, one, one, one, None, 0, 16, 16, 100, None) == 2
+    assert lib.fp8bs_gemm(None, one, one, one, one, None, 0, 16, 16, 128, None) == 1
+    assert lib.fp8bs_gemm(one, one, one, one, one, None, 0, -1, 16, 128, None) == 2
+    assert lib.fp8bs_gemm(one, one, one, one, one, None, 0, 0, 16, 128, None) == 0       # empty: nothing to do
+    assert lib.fp8bs_gemm(one, one, one, one, one, None, 0, 1 << 20, 16, 1 << 13, None) == 4   # 2^33 bytes of a
+    assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 16, 16, 128, 99, 1, None) == 7
+    assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 130, 16, 128, 2, 1, None) == 7  # tiled variant needs m%16==0
+    assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 64, 256, 1024, 4, 4, None) == 3 # split-K without workspace
+    assert lib.fp8bs_gemm_grouped(one, one, one, one, one, None, 4, 16, 16, 128, None) == 1
+    assert lib.fp8bs_gemm_grouped(one, one, one, one, one, one, 0, 16, 16, 128, None) == 6
+    for code in range(0, 9):
+        assert len(lib.fp8bs_strerror(code)) > 0
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        pkg._lib.check(2)
+
+
+def test_custom_kernel_validates_its_operands(pkg):
+    a, b, a_scale, b_scale, c = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0], m=32, n=128, k=128)
+    with pytest.raises(ValueError, match="GPU tensor"):
+        pkg.custom_kernel((a, b, a_scale, b_scale, c))           # CPU tensors: no CPU path exists
+    with pytest.raises(TypeError):
+        pkg.custom_kernel((a.float(), b, a_scale, b_scale, c))
+    with pytest.raises(TypeError):
+        pkg.custom_kernel((a, b, a_scale, b_scale, c.float()))
+
+
+def test_root_submission_module_reexports_entry_point(pkg):
+    import submission
+    assert submission.custom_kernel is pkg.custom_kernel
