@@ -26,6 +26,7 @@
 #include <stdint.h>
 #include <stddef.h>
 #include <type_traits>
+#include <utility>
 
 #include "fp8bs_kernels.h"
 
@@ -199,6 +200,19 @@ void gemm_tr_kernel(const GemmArgs p) {
     // stage and would otherwise make every LDS read wait for all outstanding copies.  Completion is
     // enforced by hand: s_waitcnt vmcnt(0) + workgroup barrier before the first read of a stage.
     const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    // one of the A_LOADS + B_LOADS copies of a block (compile-time index q) into `stage`
+    auto issue_one = [&](int stage, auto q_tag) {
+        constexpr int q = decltype(q_tag)::value;
+        const uint32_t sa = lds_base + stage * C::STAGE_BYTES + wave * 1024;
+        if constexpr (q < C::A_LOADS) {
+            copy16_global_to_lds(a_rsrc, sa + q * C::NWAVES * 1024, a_goff[q]);
+            a_goff[q] += a_kstep;
+        } else {
+            constexpr int qb = q - C::A_LOADS;
+            copy16_global_to_lds(b_rsrc, sa + C::A_BYTES + qb * C::NWAVES * 1024, b_goff[qb]);
+            b_goff[qb] += b_kstep;
+        }
+    };
     auto issue_loads = [&](int stage) {
         const uint32_t sa = lds_base + stage * C::STAGE_BYTES + wave * 1024;
         const uint32_t sb = sa + C::A_BYTES;
@@ -270,7 +284,6 @@ void gemm_tr_kernel(const GemmArgs p) {
         bs_cur = bs_row[nblk];
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
         __syncthreads();
-        if (nkb > 1) issue_loads(1);
 
         v8i areg[C::MT], breg[2];
 #pragma unroll
@@ -279,11 +292,17 @@ void gemm_tr_kernel(const GemmArgs p) {
 
         constexpr int STEPS = C::MT * C::NT;
         constexpr int LAG = 3, RING = 4;      // fold the result of step s-LAG while step s runs
+        constexpr int NLOADS = C::A_LOADS + C::B_LOADS;
+        // the copies of the next block are issued one per DMA_EVERY steps, all before the barrier step
+        constexpr int DMA_EVERY = (STEPS - C::MT) / NLOADS >= 2 ? 2 : 1, DMA_FIRST = DMA_EVERY - 1;
+        static_assert(NLOADS * DMA_EVERY <= STEPS - C::MT, "not enough steps to issue the copies before the barrier");
 
         // One K block.  HAS_NEXT is a compile-time flag so that the step sequence below is a single
         // straight-line block for the instruction scheduler.
-        auto k_block = [&](const unsigned char* sbase, const unsigned char* snext, auto has_next_tag) {
+        auto k_block = [&](int cur_stage, auto has_next_tag) {
             constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
+            const unsigned char* sbase = lds + cur_stage * C::STAGE_BYTES;
+            const unsigned char* snext = lds + (cur_stage ^ 1) * C::STAGE_BYTES;
             float sc[C::MT];
 #pragma unroll
             for (int t = 0; t < C::MT; t++) sc[t] = as_cur[t] * bs_cur;
@@ -294,12 +313,18 @@ void gemm_tr_kernel(const GemmArgs p) {
                 bs_cur = bs_row[nblk];
             }
             v4f ring[RING];
-#pragma unroll
-            for (int s = 0; s < STEPS + LAG; s++) {
-                if (s < STEPS) {
-                    const int u = s / C::MT, t = s % C::MT;
-                    if (t == 0 && u + 1 < C::NT) read_b(breg[(u + 1) & 1], u + 1, sbase);
-                    if (t == 0 && u == C::NT - 1) {
+            auto step = [&](auto s_tag) {
+                constexpr int s = decltype(s_tag)::value;
+                if constexpr (s < STEPS) {
+                    constexpr int u = s / C::MT, t = s % C::MT;
+                    // The copy of the next block into the other stage (free since the previous
+                    // barrier) is trickled out one instruction every DMA_EVERY steps: a burst of
+                    // copies would block this wave's instruction issue until the texture unit has
+                    // taken them all, and with it the MFMAs queued behind.
+                    if constexpr (HAS_NEXT && s % DMA_EVERY == DMA_FIRST && s / DMA_EVERY < NLOADS)
+                        issue_one(cur_stage ^ 1, std::integral_constant<int, s / DMA_EVERY>{});
+                    if constexpr (t == 0 && u + 1 < C::NT) read_b(breg[(u + 1) & 1], u + 1, sbase);
+                    if constexpr (t == 0 && u == C::NT - 1) {
                         // All reads of this stage are issued.  Wait for them and for this wave's part
                         // of the next block, then meet the other waves: after the barrier the next
                         // block is complete in the other stage and this stage may be overwritten.
@@ -308,31 +333,27 @@ void gemm_tr_kernel(const GemmArgs p) {
                     }
                     const v4f z = {0.f, 0.f, 0.f, 0.f};
                     ring[s % RING] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(breg[u & 1], areg[t], z, 0, 0, 0, 0, 0, 0);
-                    if (u == C::NT - 1 && HAS_NEXT) {
+                    if constexpr (u == C::NT - 1 && HAS_NEXT) {
                         // operands of the next block, fetched while the last MFMAs of this one run
                         read_a(areg[t], t, snext);
-                        if (t == 0) read_b(breg[0], 0, snext);
+                        if constexpr (t == 0) read_b(breg[0], 0, snext);
                     }
                 }
-                if (s >= LAG) {
-                    const int sp = s - LAG, u = sp / C::MT, t = sp % C::MT;
+                if constexpr (s >= LAG) {
+                    constexpr int sp = s - LAG, u = sp / C::MT, t = sp % C::MT;
 #pragma unroll
                     for (int r = 0; r < 4; r++) acc[t][u][r] = __builtin_fmaf(ring[sp % RING][r], sc[t], acc[t][u][r]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-            }
+            };
+            [&]<int... S>(std::integer_sequence<int, S...>) {
+                (step(std::integral_constant<int, S>{}), ...);
+            }(std::make_integer_sequence<int, STEPS + LAG>{});
         };
 
         int i = 0;
-        for (; i + 1 < nkb; i++) {
-            k_block(lds + (i & 1) * C::STAGE_BYTES, lds + ((i & 1) ^ 1) * C::STAGE_BYTES, std::true_type{});
-            // Block i+2 goes into the stage just released.  Issued unconditionally to keep the loop
-            // a single basic block: past the end of K the buffer bounds make the copy read zeros (or,
-            // for a K split, the next split's bytes) into a stage nobody reads again, and the final
-            // block below waits for all copies before the workgroup ends.
-            issue_loads(i & 1);
-        }
-        k_block(lds + (i & 1) * C::STAGE_BYTES, lds, std::false_type{});
+        for (; i + 1 < nkb; i++) k_block(i & 1, std::true_type{});
+        k_block(i & 1, std::false_type{});
     }
 
     // ---- epilogue -----------------------------------------------------------------------------
