@@ -52,11 +52,16 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 }
 
 // 16 bytes per lane, global -> LDS without passing through registers (buffer_load_dwordx4 ... lds):
-// lane l's bytes land at lds_base + 16*l, lds_base must be wave-uniform; lanes whose offset is beyond
-// the buffer's size read zeros.
-__device__ __forceinline__ void copy16_global_to_lds(__amdgpu_buffer_rsrc_t rsrc, uint32_t lds_base, uint32_t byte_offset) {
-    asm volatile("s_mov_b32 m0, %2\n\tbuffer_load_dwordx4 %0, %1, 0 offen lds"
-                 :: "v"(byte_offset), "s"(rsrc), "s"(lds_base) : "memory", "m0");
+// lane l's bytes land at lds_base + 16*l; lds_base and wave_offset must be wave-uniform (SGPRs), the
+// address is buffer base + lane_offset + wave_offset.
+__device__ __forceinline__ void copy16_global_to_lds(__amdgpu_buffer_rsrc_t rsrc, uint32_t lds_base, uint32_t lane_offset, uint32_t wave_offset) {
+    asm volatile("s_mov_b32 m0, %2\n\tbuffer_load_dwordx4 %0, %1, %3 offen lds"
+                 :: "v"(lane_offset), "s"(rsrc), "s"(lds_base), "s"(wave_offset) : "memory", "m0");
+}
+// same with 4 bytes per lane: lane l's dword lands at lds_base + 4*l
+__device__ __forceinline__ void copy4_global_to_lds(__amdgpu_buffer_rsrc_t rsrc, uint32_t lds_base, uint32_t lane_offset, uint32_t wave_offset) {
+    asm volatile("s_mov_b32 m0, %2\n\tbuffer_load_dword %0, %1, %3 offen lds"
+                 :: "v"(lane_offset), "s"(rsrc), "s"(lds_base), "s"(wave_offset) : "memory", "m0");
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -100,7 +105,8 @@ struct TileCfg {
     static constexpr int MT = WM / 16, NT = WN / 16;
     static constexpr int CPR_A = BM / 16, CPR_B = BN / 16;          // 16-byte chunks per k row
     static constexpr int A_BYTES = KBLK * BM, B_BYTES = KBLK * BN;
-    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+    static constexpr int AS_BYTES = BM * 4;                          // the k block's a_scale row
+    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + (AS_BYTES < 1024 ? 1024 : AS_BYTES);
     static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
     static constexpr int A_LOADS = A_BYTES / 16 / NTHREADS;         // 16-byte loads per thread per block
     static constexpr int B_LOADS = B_BYTES / 16 / NTHREADS;
@@ -175,24 +181,36 @@ void gemm_tr_kernel(const GemmArgs p) {
     __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, a_bytes, 0x00020000);
     __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)bptr, 0, b_bytes, 0x00020000);
 
-    // ---- global -> LDS copy plan: wave w, instruction i fills 1 KiB of LDS starting at chunk slot
-    //      (i*NWAVES + w)*64; lane l fills slot P = that + l.  Slot P holds k row P/CPR, stored chunk
-    //      P%CPR, which is logical chunk (P%CPR) ^ swz(k row): pick the global address accordingly.
-    uint32_t a_goff[C::A_LOADS], b_goff[C::B_LOADS];
-#pragma unroll
-    for (int i = 0; i < C::A_LOADS; i++) {
-        int P = (i * C::NWAVES + wave) * 64 + lane;
-        int krow = P / C::CPR_A, cs = P % C::CPR_A;
-        int c = cs ^ swz_of_krow<C::CPR_A>(krow);
-        a_goff[i] = (uint32_t)(kb_begin * KBLK + krow) * (uint32_t)p.lda + (uint32_t)(m0 + 16 * c);
+    // ---- global -> LDS copy plan --------------------------------------------------------------
+    // Wave w, copy q fills the 1 KiB of LDS that starts at chunk slot (q*NWAVES + w)*64; lane l fills
+    // slot P = that + l, which holds k row P/CPR, stored chunk P%CPR = logical chunk (P%CPR) ^ swz(k row).
+    // The XOR mask of a lane does not depend on q, so a lane's global offset is one constant (k row of
+    // copy 0, chunk column) plus a wave-uniform term (k block and q), which travels in an SGPR.
+    // Chunk columns beyond the matrix are clamped to its last 16 rows: such rows are never stored,
+    // and every address the copies form stays inside the operand.
+    constexpr int ROWS_PER_COPY_A = C::NWAVES * 64 / C::CPR_A, ROWS_PER_COPY_B = C::NWAVES * 64 / C::CPR_B;
+    uint32_t a_voff, b_voff;
+    {
+        int P = wave * 64 + lane;
+        int krow = P / C::CPR_A, c = (P % C::CPR_A) ^ swz_of_krow<C::CPR_A>(krow);
+        int col = m0 + 16 * c;
+        col = col < p.lda - 16 ? col : p.lda - 16;
+        a_voff = (uint32_t)krow * (uint32_t)p.lda + (uint32_t)col;
+        krow = P / C::CPR_B; c = (P % C::CPR_B) ^ swz_of_krow<C::CPR_B>(krow);
+        col = n0 + 16 * c;
+        col = col < p.n - 16 ? col : p.n - 16;
+        b_voff = (uint32_t)krow * (uint32_t)p.n + (uint32_t)col;
     }
-#pragma unroll
-    for (int i = 0; i < C::B_LOADS; i++) {
-        int P = (i * C::NWAVES + wave) * 64 + lane;
-        int krow = P / C::CPR_B, cs = P % C::CPR_B;
-        int c = cs ^ swz_of_krow<C::CPR_B>(krow);
-        b_goff[i] = (uint32_t)(kb_begin * KBLK + krow) * (uint32_t)p.n + (uint32_t)(n0 + 16 * c);
+    // a_scale row of a k block: BM floats, copied 64 floats (one dword per lane) per wave by the first
+    // BM/64 waves into the tail of the stage
+    constexpr int AS_COPIES = BM / 64;
+    uint32_t as_voff;
+    {
+        int r = m0 + wave * 64 + lane;
+        r = r < p.lda - 1 ? r : p.lda - 1;
+        as_voff = (uint32_t)r * 4u;
     }
+    __amdgpu_buffer_rsrc_t as_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.as, 0, (uint32_t)(p.k / KBLK) * (uint32_t)p.lda * 4u, 0x00020000);
     const uint32_t a_kstep = (uint32_t)KBLK * (uint32_t)p.lda, b_kstep = (uint32_t)KBLK * (uint32_t)p.n;
 
     // The copies are issued from inline assembly so that the compiler's hazard tracking does not see
@@ -200,32 +218,26 @@ void gemm_tr_kernel(const GemmArgs p) {
     // stage and would otherwise make every LDS read wait for all outstanding copies.  Completion is
     // enforced by hand: s_waitcnt vmcnt(0) + workgroup barrier before the first read of a stage.
     const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
-    // one of the A_LOADS + B_LOADS copies of a block (compile-time index q) into `stage`
-    auto issue_one = [&](int stage, auto q_tag) {
+    constexpr int NLOADS = C::A_LOADS + C::B_LOADS + 1;     // + the a_scale row
+    // copy q (compile-time) of k block `blk` (relative to kb_begin) into `stage`
+    auto issue_one = [&](int stage, int blk, auto q_tag) {
         constexpr int q = decltype(q_tag)::value;
         const uint32_t sa = lds_base + stage * C::STAGE_BYTES + wave * 1024;
+        const uint32_t kb = (uint32_t)(kb_begin + blk);
         if constexpr (q < C::A_LOADS) {
-            copy16_global_to_lds(a_rsrc, sa + q * C::NWAVES * 1024, a_goff[q]);
-            a_goff[q] += a_kstep;
-        } else {
+            copy16_global_to_lds(a_rsrc, sa + q * C::NWAVES * 1024, a_voff, kb * a_kstep + (uint32_t)(q * ROWS_PER_COPY_A) * (uint32_t)p.lda);
+        } else if constexpr (q < C::A_LOADS + C::B_LOADS) {
             constexpr int qb = q - C::A_LOADS;
-            copy16_global_to_lds(b_rsrc, sa + C::A_BYTES + qb * C::NWAVES * 1024, b_goff[qb]);
-            b_goff[qb] += b_kstep;
+            copy16_global_to_lds(b_rsrc, sa + C::A_BYTES + qb * C::NWAVES * 1024, b_voff, kb * b_kstep + (uint32_t)(qb * ROWS_PER_COPY_B) * (uint32_t)p.n);
+        } else {
+            if (wave < AS_COPIES)
+                copy4_global_to_lds(as_rsrc, lds_base + stage * C::STAGE_BYTES + C::A_BYTES + C::B_BYTES + wave * 256, as_voff, kb * (uint32_t)p.lda * 4u);
         }
     };
-    auto issue_loads = [&](int stage) {
-        const uint32_t sa = lds_base + stage * C::STAGE_BYTES + wave * 1024;
-        const uint32_t sb = sa + C::A_BYTES;
-#pragma unroll
-        for (int i = 0; i < C::A_LOADS; i++) {
-            copy16_global_to_lds(a_rsrc, sa + i * C::NWAVES * 1024, a_goff[i]);
-            a_goff[i] += a_kstep;
-        }
-#pragma unroll
-        for (int i = 0; i < C::B_LOADS; i++) {
-            copy16_global_to_lds(b_rsrc, sb + i * C::NWAVES * 1024, b_goff[i]);
-            b_goff[i] += b_kstep;
-        }
+    auto issue_all = [&](int stage, int blk) {
+        [&]<int... Q>(std::integer_sequence<int, Q...>) {
+            (issue_one(stage, blk, std::integral_constant<int, Q>{}), ...);
+        }(std::make_integer_sequence<int, NLOADS>{});
     };
 
     // ---- per-lane LDS read addresses -----------------------------------------------------------
@@ -255,14 +267,10 @@ void gemm_tr_kernel(const GemmArgs p) {
     };
 
     // ---- scales -------------------------------------------------------------------------------
-    // lane's output row for m-tile t is  m0 + wave_m*WM + 16t + i16 ; clamp so tail lanes stay in range
-    uint32_t as_off[C::MT];
-#pragma unroll
-    for (int t = 0; t < C::MT; t++) {
-        int r = m0 + wave_m * WM + 16 * t + i16;
-        r = r < p.lda - 1 ? r : p.lda - 1;
-        as_off[t] = (uint32_t)r;
-    }
+    // a_scale: lane's output row of m-tile t is tile row wave_m*WM + 16t + i16, read from the stage's
+    // copy of the a_scale row.  b_scale: one value per wave and k block (a wave's n range lies inside
+    // one 128-block), loaded straight from memory two k blocks ahead.
+    const int as_lane_off = C::A_BYTES + C::B_BYTES + (wave_m * WM + i16) * 4;
     int nblk = (n0 + wave_n * WN) / 128;
     nblk = __builtin_amdgcn_readfirstlane(nblk < p.nb - 1 ? nblk : p.nb - 1);
 
@@ -274,55 +282,54 @@ void gemm_tr_kernel(const GemmArgs p) {
 
     const int nkb = kb_end - kb_begin;
     if (nkb > 0) {
-        // ---- prologue: block 0 -> stage 0, wait, then block 1 -> stage 1 in the background ----
-        const float* as_row = p.as + (size_t)kb_begin * p.lda;     // a_scale row of the current k block
-        const float* bs_row = bsptr + (size_t)kb_begin * p.nb;
-        float as_cur[C::MT], bs_cur;
-        issue_loads(0);
-#pragma unroll
-        for (int t = 0; t < C::MT; t++) as_cur[t] = as_row[as_off[t]];
-        bs_cur = bs_row[nblk];
+        constexpr int STEPS = C::MT * C::NT;
+        constexpr int LAG = 3, RING = 4;      // fold the result of step s-LAG while step s runs
+        // Copies of block j+2 start right behind the barrier of block j (NL_LATE of them, one per
+        // trailing step) and continue one every DMA_EVERY steps of block j+1: a burst would block this
+        // wave's instruction issue until the texture unit has taken it, and the MFMAs queued behind.
+        constexpr int NL_LATE = C::MT < 2 ? C::MT : 2;
+        constexpr int NL_EARLY = NLOADS - NL_LATE;
+        constexpr int DMA_EVERY = (STEPS - C::MT) / NL_EARLY >= 2 ? 2 : 1, DMA_FIRST = DMA_EVERY - 1;
+        static_assert(NL_EARLY * DMA_EVERY <= STEPS - C::MT, "not enough steps to issue the copies before the barrier");
+
+        // ---- prologue: block 0 -> stage 0, wait; first copies of block 1 -> stage 1 ----
+        const float* bs_ptr = bsptr + (size_t)kb_begin * p.nb + nblk;   // b_scale of the current k block
+        float bs_cur = bs_ptr[0];
+        float bs_nxt = nkb > 1 ? bs_ptr[p.nb] : 0.f;
+        issue_all(0, 0);
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
         __syncthreads();
+        if (nkb > 1) {
+            [&]<int... Q>(std::integer_sequence<int, Q...>) {
+                (issue_one(1, 1, std::integral_constant<int, Q>{}), ...);
+            }(std::make_integer_sequence<int, NL_LATE>{});
+        }
 
         v8i areg[C::MT], breg[2];
 #pragma unroll
         for (int t = 0; t < C::MT; t++) read_a(areg[t], t, lds);
         read_b(breg[0], 0, lds);
 
-        constexpr int STEPS = C::MT * C::NT;
-        constexpr int LAG = 3, RING = 4;      // fold the result of step s-LAG while step s runs
-        constexpr int NLOADS = C::A_LOADS + C::B_LOADS;
-        // the copies of the next block are issued one per DMA_EVERY steps, all before the barrier step
-        constexpr int DMA_EVERY = (STEPS - C::MT) / NLOADS >= 2 ? 2 : 1, DMA_FIRST = DMA_EVERY - 1;
-        static_assert(NLOADS * DMA_EVERY <= STEPS - C::MT, "not enough steps to issue the copies before the barrier");
-
-        // One K block.  HAS_NEXT is a compile-time flag so that the step sequence below is a single
-        // straight-line block for the instruction scheduler.
-        auto k_block = [&](int cur_stage, auto has_next_tag) {
-            constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
+        // One K block (index j, in stage j&1).  The flags are compile-time so that the step sequence
+        // is one straight-line block for the instruction scheduler.
+        auto k_block = [&](int j, auto has_next_tag, auto has_next2_tag) {
+            constexpr bool HAS_NEXT = decltype(has_next_tag)::value;      // block j+1 exists
+            constexpr bool HAS_NEXT2 = decltype(has_next2_tag)::value;    // block j+2 exists
+            const int cur_stage = j & 1;
             const unsigned char* sbase = lds + cur_stage * C::STAGE_BYTES;
             const unsigned char* snext = lds + (cur_stage ^ 1) * C::STAGE_BYTES;
             float sc[C::MT];
 #pragma unroll
-            for (int t = 0; t < C::MT; t++) sc[t] = as_cur[t] * bs_cur;
-            if (HAS_NEXT) {
-                as_row += p.lda; bs_row += p.nb;
-#pragma unroll
-                for (int t = 0; t < C::MT; t++) as_cur[t] = as_row[as_off[t]];
-                bs_cur = bs_row[nblk];
-            }
+            for (int t = 0; t < C::MT; t++) sc[t] = *(const float*)(sbase + as_lane_off + t * 64) * bs_cur;
+            bs_cur = bs_nxt;
+            if constexpr (HAS_NEXT2) bs_nxt = bs_ptr[(size_t)(j + 2) * p.nb];
             v4f ring[RING];
             auto step = [&](auto s_tag) {
                 constexpr int s = decltype(s_tag)::value;
                 if constexpr (s < STEPS) {
                     constexpr int u = s / C::MT, t = s % C::MT;
-                    // The copy of the next block into the other stage (free since the previous
-                    // barrier) is trickled out one instruction every DMA_EVERY steps: a burst of
-                    // copies would block this wave's instruction issue until the texture unit has
-                    // taken them all, and with it the MFMAs queued behind.
-                    if constexpr (HAS_NEXT && s % DMA_EVERY == DMA_FIRST && s / DMA_EVERY < NLOADS)
-                        issue_one(cur_stage ^ 1, std::integral_constant<int, s / DMA_EVERY>{});
+                    if constexpr (HAS_NEXT && s % DMA_EVERY == DMA_FIRST && s / DMA_EVERY < NL_EARLY)
+                        issue_one(cur_stage ^ 1, j + 1, std::integral_constant<int, NL_LATE + s / DMA_EVERY>{});
                     if constexpr (t == 0 && u + 1 < C::NT) read_b(breg[(u + 1) & 1], u + 1, sbase);
                     if constexpr (t == 0 && u == C::NT - 1) {
                         // All reads of this stage are issued.  Wait for them and for this wave's part
@@ -338,6 +345,8 @@ void gemm_tr_kernel(const GemmArgs p) {
                         read_a(areg[t], t, snext);
                         if constexpr (t == 0) read_b(breg[0], 0, snext);
                     }
+                    if constexpr (u == C::NT - 1 && HAS_NEXT2 && t < NL_LATE)
+                        issue_one(cur_stage, j + 2, std::integral_constant<int, t>{});
                 }
                 if constexpr (s >= LAG) {
                     constexpr int sp = s - LAG, u = sp / C::MT, t = sp % C::MT;
@@ -351,9 +360,10 @@ void gemm_tr_kernel(const GemmArgs p) {
             }(std::make_integer_sequence<int, STEPS + LAG>{});
         };
 
-        int i = 0;
-        for (; i + 1 < nkb; i++) k_block(i & 1, std::true_type{});
-        k_block(i & 1, std::false_type{});
+        int j = 0;
+        for (; j + 2 < nkb; j++) k_block(j, std::true_type{}, std::true_type{});
+        if (j + 1 < nkb) { k_block(j, std::true_type{}, std::false_type{}); j++; }
+        k_block(j, std::false_type{}, std::false_type{});
     }
 
     // ---- epilogue -----------------------------------------------------------------------------
