@@ -15,7 +15,7 @@ EXPORTS = (
     "fp8bs_gemm", "fp8bs_gemm_ex", "fp8bs_gemm_grouped",
 )
 
-VARIANT_NAMES = {0: "auto", 1: "generic", 2: "t256x256", 3: "t128x128", 4: "t64x128", 5: "t256x128"}
+VARIANT_NAMES = {0: "auto", 1: "generic", 2: "t256x256", 3: "t128x128", 4: "t64x128", 5: "t256x128", 6: "skinny64x144"}
 
 
 class Plan(ctypes.Structure):

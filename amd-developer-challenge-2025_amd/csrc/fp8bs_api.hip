@@ -25,6 +25,7 @@ bool variant_info(int variant, VariantInfo* out) {
         case FP8BS_VARIANT_T128x128: *out = {128, 128, 256}; return true;
         case FP8BS_VARIANT_T64x128:  *out = {64, 128, 256}; return true;
         case FP8BS_VARIANT_T256x128: *out = {256, 128, 512}; return true;
+        case FP8BS_VARIANT_SKINNY64x144: *out = {64, 144, 256}; return true;
         default: return false;
     }
 }
@@ -63,9 +64,23 @@ void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     int kbt = k / KBLK;
     long t256 = cdiv(m, 256) * cdiv(n, 256);
     long t128 = cdiv(m, 128) * cdiv(n, 128);
-    if (m > 64 && t256 * 10 >= (long)num_cus * 9) { fill_plan(m, n, k, FP8BS_VARIANT_T256x256, 1, out); return; }
-    if (m > 64 && t128 >= num_cus) { fill_plan(m, n, k, FP8BS_VARIANT_T128x128, 1, out); return; }
-    int variant = m <= 64 ? FP8BS_VARIANT_T64x128 : FP8BS_VARIANT_T128x128;
+    if (m > 128 && t256 * 10 >= (long)num_cus * 9) { fill_plan(m, n, k, FP8BS_VARIANT_T256x256, 1, out); return; }
+    if (m > 128 && t128 >= num_cus) { fill_plan(m, n, k, FP8BS_VARIANT_T128x128, 1, out); return; }
+    if (m <= 128) {
+        // Bandwidth-bound family: stream B once with the 64x144 ring kernel.  Pick the K split that
+        // minimises (rounds over the CUs) x (K blocks per workgroup) x (bytes of B per workgroup and
+        // K block) plus the fp32 partial planes the split writes and reads back.
+        long tiles = cdiv(m, 64) * cdiv(n, 144);
+        double best = 0; int best_s = 1;
+        for (int s = 1; s <= 8 && s <= kbt; s++) {
+            double t_main = (double)cdiv(tiles * s, num_cus) * (double)cdiv(kbt, s) * 144.0 * 128.0;
+            double t_red = s > 1 ? 8.0 * s * (double)m * (double)n / num_cus : 0.0;
+            if (s == 1 || t_main + t_red < best) { best = t_main + t_red; best_s = s; }
+        }
+        fill_plan(m, n, k, FP8BS_VARIANT_SKINNY64x144, best_s, out);
+        return;
+    }
+    int variant = FP8BS_VARIANT_T128x128;
     VariantInfo vi{};
     variant_info(variant, &vi);
     long tiles = cdiv(m, vi.bm) * cdiv(n, vi.bn);

@@ -389,6 +389,186 @@ void gemm_tr_kernel(const GemmArgs p) {
 }
 
 // ---------------------------------------------------------------------------------------------------
+// Skinny-M streaming kernel (bandwidth-bound shapes: a few rows of A against a long B).
+//
+// One workgroup = 64 rows of A x 144 columns of B over a K range; 4 waves.  The work per K block is
+// tiny, the time goes into streaming B from HBM once, so the design is a deep ring of LDS stages kept
+// full by asynchronous global->LDS copies: NSTAGE = 5 stages of (A 8 KiB + B 18 KiB + scales), four K
+// blocks in flight per workgroup, one barrier per K block.  144 = 9 sixteen-byte chunks: with an odd
+// number of chunks per k row the 16 k rows a transposing read touches already fall on 16 different bank
+// groups, so the B tile needs no swizzle; and 18432 / 144 = 128 tiles x split-K 2 fills 256 CUs exactly.
+// Every wave issues the same number of copies per block (7), which makes "block j has landed" a fixed
+// s_waitcnt vmcnt threshold.  The scales of the block (a_scale row, the <= 3 b_scale values the 144
+// columns span) ride the same ring.
+//   MODE 0: bf16 output      MODE 1: fp32 split-K partial planes
+// ---------------------------------------------------------------------------------------------------
+struct SkinnyCfg {
+    static constexpr int BM = 64, BN = 144, CPR_A = 4, CPR_B = 9, NWAVES = 4, NTHREADS = 256;
+    static constexpr int A_BYTES = KBLK * BM, B_BYTES = KBLK * BN, SC_BYTES = 1024;
+    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + SC_BYTES;      // 27 KiB
+    static constexpr int NSTAGE = 5;
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;               // 135 KiB
+    static constexpr int COPIES = 7;                                      // per wave per K block
+    static constexpr int MT = BM / 16, NT_MAX = 3;                        // n tiles per wave: ceil(9 / 4)
+    static_assert(A_BYTES / 1024 + B_BYTES / 1024 + 2 == COPIES * NWAVES, "copy plan must cover a block exactly");
+};
+
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    // s_waitcnt with only vmcnt constrained: vmcnt is split over bits [3:0] and [15:14]
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256)
+void gemm_skinny_kernel(const GemmArgs p) {
+    using C = SkinnyCfg;
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 4, i16 = lane & 15;
+
+    const int tiles_n = (p.n + C::BN - 1) / C::BN;
+    // neighbouring n tiles share 128-byte lines of every k row of B (144 is not a multiple of 128):
+    // give each XCD a contiguous run of tiles so that the shared lines are fetched into one L2 only
+    const int bid = xcd_virtual_id(blockIdx.x, gridDim.x);
+    const int tn = bid % tiles_n, split_z = (bid / tiles_n) % p.split_k, tm = bid / (tiles_n * p.split_k);
+    const int m0 = tm * C::BM, n0 = tn * C::BN;
+    const int kbt = p.k / KBLK;
+    const int kb_begin = split_z * p.kb_per_split;
+    int kb_end = kb_begin + p.kb_per_split;
+    kb_end = kb_end < kbt ? kb_end : kbt;
+    const int nkb = kb_end - kb_begin;
+    const int nb0 = n0 / 128;
+
+    __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, (uint32_t)p.k * (uint32_t)p.lda, 0x00020000);
+    __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.b, 0, (uint32_t)p.k * (uint32_t)p.n, 0x00020000);
+    __amdgpu_buffer_rsrc_t as_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.as, 0, (uint32_t)kbt * (uint32_t)p.lda * 4u, 0x00020000);
+    __amdgpu_buffer_rsrc_t bs_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.bs, 0, (uint32_t)kbt * (uint32_t)p.nb * 4u, 0x00020000);
+
+    // ---- copy plan.  The 28 one-KiB copies of a block are numbered I = 4q + wave, q = 0..6:
+    //      I 0..7 the A tile, 8..25 the B tile (copy Ib = I - 8 fills B chunks 64*Ib ..), 26 the a_scale
+    //      row, 27 the b_scale values.  Lane offsets are fixed for the whole kernel; the K block enters
+    //      through the wave-uniform offset.  Columns beyond the matrix are clamped (never stored).
+    uint32_t a_voff, b_voff[5], sc_voff = 0;
+    {
+        int krow = lane / 4;                                       // + 16*I
+        int c = (lane % 4) ^ swz_of_krow<C::CPR_A>(krow);          // the XOR mask does not depend on I
+        int col = m0 + 16 * c;
+        col = col < p.lda - 16 ? col : p.lda - 16;
+        a_voff = (uint32_t)krow * (uint32_t)p.lda + (uint32_t)col;
+#pragma unroll
+        for (int i = 0; i < 5; i++) {
+            int P = 64 * (4 * i + wave) + lane;
+            int kr = P / C::CPR_B, cc = P % C::CPR_B;
+            int cl = n0 + 16 * cc;
+            cl = cl < p.n - 16 ? cl : p.n - 16;
+            b_voff[i] = (uint32_t)kr * (uint32_t)p.n + (uint32_t)cl;
+        }
+        if (wave == 2) { int r = m0 + lane; r = r < p.lda - 1 ? r : p.lda - 1; sc_voff = (uint32_t)r * 4u; }
+        if (wave == 3) { int x = nb0 + lane; x = x < p.nb - 1 ? x : p.nb - 1; sc_voff = (uint32_t)x * 4u; }
+    }
+    const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    auto issue_block = [&](int blk) {      // all 7 copies of K block `blk` (relative to kb_begin)
+        const uint32_t st = lds_base + (uint32_t)(blk % C::NSTAGE) * C::STAGE_BYTES;
+        const uint32_t kb = (uint32_t)(kb_begin + blk);
+        const uint32_t a_k = kb * (uint32_t)KBLK * (uint32_t)p.lda, b_k = kb * (uint32_t)KBLK * (uint32_t)p.n;
+        copy16_global_to_lds(a_rsrc, st + wave * 1024, a_voff, a_k + (uint32_t)(16 * wave) * (uint32_t)p.lda);
+        copy16_global_to_lds(a_rsrc, st + (4 + wave) * 1024, a_voff, a_k + (uint32_t)(16 * (4 + wave)) * (uint32_t)p.lda);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            copy16_global_to_lds(b_rsrc, st + C::A_BYTES + (4 * i + wave) * 1024, b_voff[i], b_k);
+        if (wave < 2) copy16_global_to_lds(b_rsrc, st + C::A_BYTES + (16 + wave) * 1024, b_voff[4], b_k);
+        else if (wave == 2) copy4_global_to_lds(as_rsrc, st + C::A_BYTES + C::B_BYTES, sc_voff, kb * (uint32_t)p.lda * 4u);
+        else copy4_global_to_lds(bs_rsrc, st + C::A_BYTES + C::B_BYTES + 256, sc_voff, kb * (uint32_t)p.nb * 4u);
+    };
+
+    // ---- LDS read addresses ----
+    const int krow_lane = 8 * g + (i16 >> 1);
+    const int swz_a = swz_of_krow<C::CPR_A>(krow_lane);
+    const int a_lane_off = krow_lane * C::BM + (i16 & 1) * 8;
+    const int b_lane_off = C::A_BYTES + krow_lane * C::BN + (i16 & 1) * 8;
+
+    v4f acc[C::MT][C::NT_MAX];
+#pragma unroll
+    for (int t = 0; t < C::MT; t++)
+#pragma unroll
+        for (int x = 0; x < C::NT_MAX; x++) acc[t][x] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    // ---- prologue: NSTAGE-1 blocks in flight ----
+    for (int b = 0; b < C::NSTAGE - 1 && b < nkb; b++) issue_block(b);
+
+    for (int j = 0; j < nkb; j++) {
+        // blocks issued after block j so far: up to NSTAGE-2; wait until only those are outstanding
+        int ahead = (nkb - 1 < j + C::NSTAGE - 2 ? nkb - 1 : j + C::NSTAGE - 2) - j;
+        if (ahead >= 3) wait_vmcnt<3 * C::COPIES>();
+        else if (ahead == 2) wait_vmcnt<2 * C::COPIES>();
+        else if (ahead == 1) wait_vmcnt<C::COPIES>();
+        else wait_vmcnt<0>();
+        __syncthreads();      // block j complete in LDS; everyone is done with the stage of block j-1
+        if (j + C::NSTAGE - 1 < nkb) issue_block(j + C::NSTAGE - 1);
+
+        const unsigned char* sbase = lds + (j % C::NSTAGE) * C::STAGE_BYTES;
+        const unsigned char* sc = sbase + C::A_BYTES + C::B_BYTES;
+        float asv[C::MT];
+        v8i areg[C::MT];
+#pragma unroll
+        for (int t = 0; t < C::MT; t++) {
+            asv[t] = *(const float*)(sc + (16 * t + i16) * 4);
+            const unsigned char* q = sbase + a_lane_off + ((t ^ swz_a) << 4);
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++) {
+                v2i x = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_V2I(q + jj * 32 * C::BM));
+                areg[t][2 * jj] = x[0]; areg[t][2 * jj + 1] = x[1];
+            }
+        }
+#pragma unroll
+        for (int x = 0; x < C::NT_MAX; x++) {
+            const int u = wave + 4 * x;                 // wave-uniform
+            if (u < C::CPR_B) {
+                v8i breg;
+                const unsigned char* q = sbase + b_lane_off + (u << 4);
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    v2i y = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_V2I(q + jj * 32 * C::BN));
+                    breg[2 * jj] = y[0]; breg[2 * jj + 1] = y[1];
+                }
+                int bi = ((n0 + 16 * u) >> 7) - nb0;     // which of the staged b_scale values
+                const float bsv = *(const float*)(sc + 256 + bi * 4);
+#pragma unroll
+                for (int t = 0; t < C::MT; t++) {
+                    const v4f z = {0.f, 0.f, 0.f, 0.f};
+                    v4f d = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(breg, areg[t], z, 0, 0, 0, 0, 0, 0);
+                    const float s = asv[t] * bsv;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc[t][x][r] = __builtin_fmaf(d[r], s, acc[t][x][r]);
+                }
+            }
+        }
+    }
+
+    // ---- epilogue ----
+#pragma unroll
+    for (int t = 0; t < C::MT; t++) {
+        const int row = m0 + 16 * t + i16;
+        if (row >= p.m) continue;
+#pragma unroll
+        for (int x = 0; x < C::NT_MAX; x++) {
+            const int u = wave + 4 * x;
+            const int col = n0 + 16 * u + 4 * g;
+            if (u >= C::CPR_B || col >= p.n) continue;
+            if (MODE == 1) {
+                *(v4f*)(p.ws + ((size_t)split_z * p.m + row) * (size_t)p.n + col) = acc[t][x];
+            } else {
+                v2i o;
+                o[0] = (int)pack_bf16x2(acc[t][x][0], acc[t][x][1]);
+                o[1] = (int)pack_bf16x2(acc[t][x][2], acc[t][x][3]);
+                *(v2i*)(p.c + (size_t)row * p.n + col) = o;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
 // Split-K reduction: sums `split_k` fp32 planes in a fixed order and rounds to bf16, 8 outputs per
 // thread with one 16-byte store (role of fp8_mm_128x128_ft2_split4_merge,
 // 1-amd-fp8-mm/amd-fp8-mm-submission.py:485-511, for any split count).
@@ -489,6 +669,23 @@ hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t str
         case 3: return launch_shape<128, 128, 64, 64>(a, mode, stream);
         case 4: return launch_shape<64, 128, 32, 64>(a, mode, stream);
         case 5: return launch_shape<256, 128, 64, 64>(a, mode, stream);
+        case 6: {
+            if (mode == 2) return hipErrorInvalidValue;
+            using C = SkinnyCfg;
+            auto k0 = gemm_skinny_kernel<0>;
+            auto k1 = gemm_skinny_kernel<1>;
+            static bool attr_done = false;
+            if (!attr_done) {
+                hipError_t e = hipFuncSetAttribute((const void*)k0, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+                if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+                if (e != hipSuccess) return e;
+                attr_done = true;
+            }
+            int tiles = ((a.n + C::BN - 1) / C::BN) * a.split_k * ((a.m + C::BM - 1) / C::BM);
+            if (mode == 1) hipLaunchKernelGGL(k1, dim3(tiles), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
+            else hipLaunchKernelGGL(k0, dim3(tiles), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
+            return hipGetLastError();
+        }
         default: return hipErrorInvalidValue;
     }
 }
@@ -506,6 +703,7 @@ int variant_lds_bytes(int variant) {
         case 3: return TileCfg<128, 128, 64, 64, 0>::LDS_BYTES;
         case 4: return TileCfg<64, 128, 32, 64, 0>::LDS_BYTES;
         case 5: return TileCfg<256, 128, 64, 64, 0>::LDS_BYTES;
+        case 6: return SkinnyCfg::LDS_BYTES;
         default: return 0;
     }
 }

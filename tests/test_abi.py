@@ -29,8 +29,8 @@ def test_plan_shape_families(pkg):
     p = pkg.plan(4096, 4096, 4096)
     assert p.variant == 2 and (p.tile_m, p.tile_n) == (256, 256) and p.split_k == 1 and p.workspace_bytes == 0
     assert p.grid_x == 256 and p.block_threads == 512 and p.lds_bytes == 2 * (128 * 512 + 1024)
-    p = pkg.plan(64, 18432, 7168)                       # skinny-M: small tile, split-K, workspace
-    assert p.variant == 4 and p.tile_m == 64 and p.split_k > 1
+    p = pkg.plan(64, 18432, 7168)                       # skinny-M: streaming tile, split-K fills the CUs
+    assert p.variant == 6 and (p.tile_m, p.tile_n) == (64, 144) and p.split_k == 2 and p.grid_x == 256
     assert p.workspace_bytes == p.split_k * 64 * 18432 * 4 == pkg.workspace_bytes(64, 18432, 7168)
     p = pkg.plan(130, 192, 256)                         # not a multiple of 16 -> generic kernel
     assert p.variant == 1 and p.split_k == 1
