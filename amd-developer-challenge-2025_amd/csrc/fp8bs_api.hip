@@ -56,18 +56,47 @@ void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out)
 }
 
 // Shape-family rule.  m or n not a multiple of 16 -> generic kernel (the tiled kernels copy 16-byte
-// chunks along m and n).  Otherwise pick the largest tile that still fills the chip, and split K when
-// even the smallest tile leaves most CUs idle (skinny-M, bandwidth-bound shapes).
+// chunks along m and n).  m > 128 -> the tiled MFMA kernel whose tile shape finishes soonest under a
+// small cost model.  m <= 128 -> the streaming kernel with the K split that fills the CUs.
 void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     if (num_cus <= 0) num_cus = 256;
     if ((m % 16) != 0 || (n % 16) != 0) { fill_plan(m, n, k, FP8BS_VARIANT_GENERIC, 1, out); return; }
     int kbt = k / KBLK;
-    long t256 = cdiv(m, 256) * cdiv(n, 256);
-    long t128 = cdiv(m, 128) * cdiv(n, 128);
-    if (m > 128 && t256 * 10 >= (long)num_cus * 9) { fill_plan(m, n, k, FP8BS_VARIANT_T256x256, 1, out); return; }
-    if (m > 128 && t128 >= num_cus) { fill_plan(m, n, k, FP8BS_VARIANT_T128x128, 1, out); return; }
-    if (m <= 128) {
-        // Bandwidth-bound family: stream B once with the 64x144 ring kernel.  Pick the K split that
+    if (m > 128) {
+        // Compute-bound family.  Cost model in units of "one 256x256 tile over all of K on a CU of its
+        // own": rounds over the chip x workgroups sharing a CU x tile area x a measured per-area
+        // penalty (smaller tiles re-read more of A and B from LDS per multiply).
+        struct Cand { int variant; int wgs_per_cu; double area, penalty; };
+        const Cand cands[3] = {
+            {FP8BS_VARIANT_T256x256, 1, 1.0, 1.0},
+            {FP8BS_VARIANT_T256x128, 1, 0.5, 1.16},
+            {FP8BS_VARIANT_T128x128, 2, 0.25, 1.29},
+        };
+        int best_variant = 0; double best_cost = 0;
+        for (const Cand& c : cands) {
+            VariantInfo vi{};
+            variant_info(c.variant, &vi);
+            long tiles = cdiv(m, vi.bm) * cdiv(n, vi.bn);
+            double cost = (double)cdiv(tiles, (long)num_cus * c.wgs_per_cu) * c.wgs_per_cu * c.area * c.penalty;
+            if (best_variant == 0 || cost < best_cost) { best_variant = c.variant; best_cost = cost; }
+        }
+        VariantInfo vi{};
+        variant_info(best_variant, &vi);
+        long tiles = cdiv(m, vi.bm) * cdiv(n, vi.bn);
+        // split K only when the tiles cover less than half of the chip and K is long
+        int s = 1;
+        if (tiles * 2 <= num_cus && kbt >= 8) {
+            long want = num_cus / tiles;
+            long max_split = kbt / 4;
+            s = (int)(want > max_split ? max_split : want);
+            if (s > 8) s = 8;
+            if (s < 1) s = 1;
+        }
+        fill_plan(m, n, k, best_variant, s, out);
+        return;
+    }
+    {
+        // Bandwidth-bound family (m <= 128): stream B once with the 64x144 ring kernel.  Pick the K split that
         // minimises (rounds over the CUs) x (K blocks per workgroup) x (bytes of B per workgroup and
         // K block) plus the fp32 partial planes the split writes and reads back.
         long tiles = cdiv(m, 64) * cdiv(n, 144);
@@ -78,18 +107,7 @@ void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
             if (s == 1 || t_main + t_red < best) { best = t_main + t_red; best_s = s; }
         }
         fill_plan(m, n, k, FP8BS_VARIANT_SKINNY64x144, best_s, out);
-        return;
     }
-    int variant = FP8BS_VARIANT_T128x128;
-    VariantInfo vi{};
-    variant_info(variant, &vi);
-    long tiles = cdiv(m, vi.bm) * cdiv(n, vi.bn);
-    // aim for about two workgroups per CU, keep at least 4 K blocks per split
-    long want = cdiv(2L * num_cus, tiles);
-    long max_split = kbt / 4 > 0 ? kbt / 4 : 1;
-    long s = want < 1 ? 1 : (want > max_split ? max_split : want);
-    if (s > 16) s = 16;
-    fill_plan(m, n, k, variant, (int)s, out);
 }
 
 int check_common(const void* a, const void* b, const float* as, const float* bs, void* c, int m, int n, int k) {

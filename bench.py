@@ -27,6 +27,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP8_TFLOPS = 5033.0      # 256 CU x 2.4 GHz x 8192 FLOP/clk/CU, dense e4m3
 PEAK_HBM_GBS = 8000.0
+# HBM/fabric bytes per launch of the 256x256 kernel on configuration 2, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (KiB per dispatch: 50,280 and 34,910) scaled by what the same counters read for a 128 MiB
+# device copy (`--calibrate-copy`: x2.00 and x1.00); the summary is profiles/gemm_tr_256x256_cfg2_4096cubed.txt
+TRAFFIC_CFG2_BYTES = (50280 * 2.00 + 34910 * 1.00) * 1024
 
 
 def algorithmic_bytes(m, n, k):
@@ -97,6 +101,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--configs", type=str, default="3,4,5", help="extra configurations reported under per_config")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run plain device copies of a known size (128 MiB read + 128 MiB written per copy), "
+                         "the yardstick for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the path has no multi-GPU part); run with --gpus 1", file=sys.stderr)
@@ -108,6 +115,14 @@ def main():
     pkg = importlib.import_module("amd-developer-challenge-2025_amd")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calibrate_copy:
+        srcs = [torch.full((128 * 2 ** 20,), i, dtype=torch.uint8, device=dev) for i in range(4)]   # 4 x 128 MiB > the 256 MB cache
+        dst = torch.empty_like(srcs[0])
+        for i in range(args.steps):
+            dst.copy_(srcs[i % 4])
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy": {"bytes_read_per_copy": dst.numel(), "bytes_written_per_copy": dst.numel(), "copies": args.steps}}))
+        return
     cfg2 = pkg.inputs.CONFIGS[1]
 
     # ---- headline: configuration 2, seeded CPU inputs moved to HBM before the timed region ----
@@ -141,7 +156,7 @@ def main():
         "config": {"workload": "cfg2: M=N=K=4096, A 1x128 / B 128x128 fp32 block scales, bf16 out, seed %d" % cfg2.seed,
                    "variant": pkg._lib.VARIANT_NAMES[plan.variant], "split_k": plan.split_k, "grid": plan.grid_x},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_FP8_TFLOPS, 4), "traffic": None, "us_per_launch": round(ev_us, 3)},
+                     "frac": round(achieved / PEAK_FP8_TFLOPS, 4), "traffic": TRAFFIC_CFG2_BYTES, "us_per_launch": round(ev_us, 3)},
     }
 
     # ---- other configurations ----
