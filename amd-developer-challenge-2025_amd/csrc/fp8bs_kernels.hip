@@ -393,8 +393,13 @@ void gemm_tr_kernel(const GemmArgs p) {
 //
 // One workgroup = 64 rows of A x 144 columns of B over a K range; 4 waves.  The work per K block is
 // tiny, the time goes into streaming B from HBM once, so the design is a deep ring of LDS stages kept
-// full by asynchronous global->LDS copies: NSTAGE = 5 stages of (A 8 KiB + B 18 KiB + scales), four K
-// blocks in flight per workgroup, one barrier per K block.  144 = 9 sixteen-byte chunks: with an odd
+// full by asynchronous global->LDS copies: NSTAGE = 4 stages of (A 8 KiB + B 18 KiB + scales), three K
+// blocks in flight per workgroup, one barrier per K block (a fifth stage measured slower: workgroups
+// drift further apart in K and evict the 128-byte lines they share with their neighbours from L2).
+// Split-K partial planes are summed by a separate small kernel: an in-kernel last-arriver reduction
+// was measured 1.5x slower overall, because exchanging the planes between XCDs needs either an L2
+// write-back + invalidate per workgroup (which evicts the B lines still in use) or device-coherent
+// 4-byte accesses.  144 = 9 sixteen-byte chunks: with an odd
 // number of chunks per k row the 16 k rows a transposing read touches already fall on 16 different bank
 // groups, so the B tile needs no swizzle; and 18432 / 144 = 128 tiles x split-K 2 fills 256 CUs exactly.
 // Every wave issues the same number of copies per block (7), which makes "block j has landed" a fixed
@@ -406,8 +411,8 @@ struct SkinnyCfg {
     static constexpr int BM = 64, BN = 144, CPR_A = 4, CPR_B = 9, NWAVES = 4, NTHREADS = 256;
     static constexpr int A_BYTES = KBLK * BM, B_BYTES = KBLK * BN, SC_BYTES = 1024;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + SC_BYTES;      // 27 KiB
-    static constexpr int NSTAGE = 5;
-    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;               // 135 KiB
+    static constexpr int NSTAGE = 4;
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;               // 108 KiB
     static constexpr int COPIES = 7;                                      // per wave per K block
     static constexpr int MT = BM / 16, NT_MAX = 3;                        // n tiles per wave: ceil(9 / 4)
     static_assert(A_BYTES / 1024 + B_BYTES / 1024 + 2 == COPIES * NWAVES, "copy plan must cover a block exactly");
