@@ -113,6 +113,7 @@ struct TileCfg {
     static_assert(A_BYTES % (16 * NTHREADS) == 0 && B_BYTES % (16 * NTHREADS) == 0, "tile/threads");
     static_assert(WN <= 128 && 128 % WN == 0, "a wave's n range must stay inside one b_scale block");
     static_assert(CPR_A <= 16 && CPR_B <= 16, "swizzle assumes a k row spans at most 256 bytes");
+    static_assert(BM * BN * 2 <= LDS_BYTES, "the bf16 epilogue stages the whole tile in LDS");
 };
 
 template <int CPR>
@@ -367,23 +368,51 @@ void gemm_tr_kernel(const GemmArgs p) {
     }
 
     // ---- epilogue -----------------------------------------------------------------------------
+    if (MODE == 1) {
+        // split-K: fp32 partial tile, 16 bytes per lane
 #pragma unroll
-    for (int t = 0; t < C::MT; t++) {
-        const int row = m0 + wave_m * WM + 16 * t + i16;
-        if (row < row_lo || row >= row_hi) continue;
+        for (int t = 0; t < C::MT; t++) {
+            const int row = m0 + wave_m * WM + 16 * t + i16;
+            if (row >= row_hi) continue;
 #pragma unroll
-        for (int u = 0; u < C::NT; u++) {
-            const int col = n0 + wave_n * WN + 16 * u + 4 * g;
-            if (col >= p.n) continue;
-            if (MODE == 1) {
-                float* dst = p.ws + ((size_t)split_z * p.m + row) * (size_t)p.n + col;
-                *(v4f*)dst = acc[t][u];
-            } else {
+            for (int u = 0; u < C::NT; u++) {
+                const int col = n0 + wave_n * WN + 16 * u + 4 * g;
+                if (col >= p.n) continue;
+                *(v4f*)(p.ws + ((size_t)split_z * p.m + row) * (size_t)p.n + col) = acc[t][u];
+            }
+        }
+    } else {
+        // bf16 through LDS so that the global stores are 16 bytes per lane and every store
+        // instruction writes whole rows of the wave tile (WN*2 contiguous bytes each).  The stages are
+        // free: after the barrier of the last K block no wave reads them and no copy is in flight.
+        // Each wave uses its own WM x WN bf16 region; 16-byte chunks are XOR-swizzled by row so that
+        // neither the 8-byte writes (16 rows per instruction) nor the 16-byte reads conflict.
+        constexpr int ROW_CHUNKS = WN * 2 / 16;                       // 16-byte chunks per tile row
+        constexpr int ROWS_PER_SWEEP = 16 / ROW_CHUNKS > 0 ? 16 / ROW_CHUNKS : 1;
+        unsigned char* region = lds + wave * (WM * WN * 2);
+#pragma unroll
+        for (int t = 0; t < C::MT; t++) {
+            const int r = 16 * t + i16;
+            const int sw = (r / ROWS_PER_SWEEP) % ROW_CHUNKS;
+#pragma unroll
+            for (int u = 0; u < C::NT; u++) {
                 v2i o;
                 o[0] = (int)pack_bf16x2(acc[t][u][0], acc[t][u][1]);
                 o[1] = (int)pack_bf16x2(acc[t][u][2], acc[t][u][3]);
-                *(v2i*)(p.c + (size_t)row * p.n + col) = o;
+                const int chunk = 2 * u + (g >> 1);
+                *(v2i*)(region + r * (WN * 2) + ((chunk ^ sw) << 4) + (g & 1) * 8) = o;
             }
+        }
+        constexpr int PASSES = WM * ROW_CHUNKS / 64;
+#pragma unroll
+        for (int q = 0; q < PASSES; q++) {
+            const int idx = q * 64 + lane;
+            const int r = idx / ROW_CHUNKS, chunk = idx % ROW_CHUNKS;
+            const int sw = (r / ROWS_PER_SWEEP) % ROW_CHUNKS;
+            const v4i val = *(const v4i*)(region + r * (WN * 2) + ((chunk ^ sw) << 4));
+            const int row = m0 + wave_m * WM + r, col = n0 + wave_n * WN + chunk * 8;
+            if (row >= row_lo && row < row_hi && col < p.n)
+                *(v4i*)(p.c + (size_t)row * p.n + col) = val;
         }
     }
 }
