@@ -202,12 +202,15 @@ void gemm_tr_kernel(const GemmArgs p) {
         col = col < p.n - 16 ? col : p.n - 16;
         b_voff = (uint32_t)krow * (uint32_t)p.n + (uint32_t)col;
     }
-    // a_scale row of a k block: BM floats, copied 64 floats (one dword per lane) per wave by the first
-    // BM/64 waves into the tail of the stage
+    // a_scale row of a k block: BM floats, copied 64 floats (one dword per lane) per wave into the tail
+    // of the stage.  Every wave issues the copy (wave w the same 64 floats as wave w % (BM/64), to the
+    // same place): a branch here would split the K loop's straight-line block and the compiler would
+    // sink the folds of the first MFMAs below it, away from the MFMAs they are meant to overlap.
     constexpr int AS_COPIES = BM / 64;
+    const int as_wave = wave % AS_COPIES;
     uint32_t as_voff;
     {
-        int r = m0 + wave * 64 + lane;
+        int r = m0 + as_wave * 64 + lane;
         r = r < p.lda - 1 ? r : p.lda - 1;
         as_voff = (uint32_t)r * 4u;
     }
@@ -231,8 +234,7 @@ void gemm_tr_kernel(const GemmArgs p) {
             constexpr int qb = q - C::A_LOADS;
             copy16_global_to_lds(b_rsrc, sa + C::A_BYTES + qb * C::NWAVES * 1024, b_voff, kb * b_kstep + (uint32_t)(qb * ROWS_PER_COPY_B) * (uint32_t)p.n);
         } else {
-            if (wave < AS_COPIES)
-                copy4_global_to_lds(as_rsrc, lds_base + stage * C::STAGE_BYTES + C::A_BYTES + C::B_BYTES + wave * 256, as_voff, kb * (uint32_t)p.lda * 4u);
+            copy4_global_to_lds(as_rsrc, lds_base + stage * C::STAGE_BYTES + C::A_BYTES + C::B_BYTES + as_wave * 256, as_voff, kb * (uint32_t)p.lda * 4u);
         }
     };
     auto issue_all = [&](int stage, int blk) {
