@@ -28,9 +28,9 @@ sys.path.insert(0, ROOT)
 PEAK_FP8_TFLOPS = 5033.0      # 256 CU x 2.4 GHz x 8192 FLOP/clk/CU, dense e4m3
 PEAK_HBM_GBS = 8000.0
 # HBM/fabric bytes per launch of the 256x256 kernel on configuration 2, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (KiB per dispatch: 50,280 and 34,910) scaled by what the same counters read for a 128 MiB
+# WRITE_SIZE (KiB per dispatch: 49,770 and 32,770) scaled by what the same counters read for a 128 MiB
 # device copy (`--calibrate-copy`: x2.00 and x1.00); the summary is profiles/gemm_tr_256x256_cfg2_4096cubed.txt
-TRAFFIC_CFG2_BYTES = (50280 * 2.00 + 34910 * 1.00) * 1024
+TRAFFIC_CFG2_BYTES = (49770 * 2.00 + 32770 * 1.00) * 1024
 
 
 def algorithmic_bytes(m, n, k):

@@ -48,7 +48,7 @@ enum {
     FP8BS_VARIANT_T128x128 = 3,   /* mid-size: 128x128 tile, 4 waves                         */
     FP8BS_VARIANT_T64x128 = 4,    /* skinny-M: 64(m) x 128(n) tile, 4 waves, split-K         */
     FP8BS_VARIANT_T256x128 = 5,   /* 256(m) x 128(n) tile, 8 waves                           */
-    FP8BS_VARIANT_SKINNY64x144 = 6, /* bandwidth-bound: 64(m) x 144(n) tile, 5-stage copy ring */
+    FP8BS_VARIANT_SKINNY64x144 = 6, /* bandwidth-bound: 64(m) x 144(n) tile, 4-stage copy ring */
     FP8BS_VARIANT_COUNT = 7
 };
 
