@@ -9,7 +9,8 @@ Layout of the package:
   build.py        compiles csrc/ into libfp8bs.so next to this file
   _lib.py         ctypes binding of the C ABI; raises if the library is missing
   submission.py   custom_kernel(data) / grouped_kernel(data): the reference's Python entry points
-  inputs.py       e4m3fn block quantisers and the synthetic inputs of the benchmark configurations
+  inputs.py       host-side e4m3fn block quantisers and the synthetic inputs of the benchmark configurations
+  quant.py        quantize_a / quantize_b: the HIP quantisers (fp32/bf16 -> operands in the GEMM's layout)
 """
 from .submission import custom_kernel, grouped_kernel, plan, workspace_bytes  # noqa: F401
 from . import inputs  # noqa: F401

@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(HERE, "libfp8bs.so")
 EXPORTS = (
     "fp8bs_version", "fp8bs_strerror", "fp8bs_plan", "fp8bs_workspace_bytes",
     "fp8bs_gemm", "fp8bs_gemm_ex", "fp8bs_gemm_grouped",
+    "fp8bs_quantize_a", "fp8bs_quantize_b",
 )
 
 VARIANT_NAMES = {0: "auto", 1: "generic", 2: "t256x256", 3: "t128x128", 4: "t64x128", 5: "t256x128", 6: "skinny64x144"}
@@ -56,6 +57,11 @@ def load() -> ctypes.CDLL:
     lib.fp8bs_gemm_ex.argtypes = [vp, vp, vp, vp, vp, vp, sz, i32, i32, i32, i32, i32, vp]
     lib.fp8bs_gemm_grouped.restype = i32
     lib.fp8bs_gemm_grouped.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]
+    i64 = ctypes.c_int64
+    lib.fp8bs_quantize_a.restype = i32
+    lib.fp8bs_quantize_a.argtypes = [vp, i32, i64, vp, i32, vp, vp, i32, i32, vp]
+    lib.fp8bs_quantize_b.restype = i32
+    lib.fp8bs_quantize_b.argtypes = [vp, i32, i64, vp, vp, i32, i32, vp]
     _lib = lib
     return lib
 

@@ -1,0 +1,66 @@
+"""GPU block quantisers: row-major fp32/bf16 matrices -> the operands ``custom_kernel`` takes.
+
+The reference has no quantiser (its operands arrive quantised, 1-amd-fp8-mm/0-amd-fp8-mm-new-begins.py:66-77);
+these wrap ``fp8bs_quantize_a`` / ``fp8bs_quantize_b`` of libfp8bs.so and return tensors with exactly
+the shapes, dtypes and K-major strides of that contract.  The rule is the one of ``inputs.quantize_a`` /
+``inputs.quantize_b`` (the host-side quantisers), bit for bit.  No fallback: without the library the
+import of ``_lib`` raises.
+"""
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _check_input(x: torch.Tensor, name: str) -> None:
+    if x.dtype not in _DTYPES:
+        raise TypeError("%s must be float32 or bfloat16, got %s" % (name, x.dtype))
+    if x.dim() != 2 or not x.is_cuda:
+        raise ValueError("%s must be a 2-D tensor on the GPU" % name)
+    if x.shape[1] % 128 != 0:
+        raise ValueError("%s: K = %d is not a multiple of 128" % (name, x.shape[1]))
+    if x.shape[1] > 0 and x.stride(1) != 1:
+        raise ValueError("%s must be row-major (stride 1 along K), got strides %s" % (name, tuple(x.stride())))
+
+
+def quantize_a(x: torch.Tensor, row_map: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """x [T, K] -> (a e4m3fn [M, K] stride (1, M), a_scale fp32 [M, K/128] stride (1, M)).
+
+    Without ``row_map`` M = T.  With ``row_map`` (int32 [M] on the GPU) output row i is input row
+    ``row_map[i]``: the expert-contiguous gather of routed tokens, fused into the quantiser.
+    """
+    _check_input(x, "x")
+    t, k = x.shape
+    if row_map is not None:
+        if row_map.dtype != torch.int32 or row_map.dim() != 1 or row_map.device != x.device or not row_map.is_contiguous():
+            raise ValueError("row_map must be a contiguous int32 vector on x's device")
+        m = row_map.numel()
+    else:
+        m = t
+    a_store = torch.empty(k, m, dtype=torch.float8_e4m3fn, device=x.device)
+    s_store = torch.empty(k // 128, m, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _lib.check(_lib.load().fp8bs_quantize_a(
+            x.data_ptr(), _DTYPES[x.dtype], x.stride(0) if t > 1 else max(k, 1),
+            row_map.data_ptr() if row_map is not None else None, t,
+            a_store.data_ptr(), s_store.data_ptr(), m, k, stream))
+    return a_store.t(), s_store.t()
+
+
+def quantize_b(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """w [N, K] -> (b e4m3fn [N, K] stride (1, N), b_scale fp32 [ceil(N/128), K/128] stride (1, NB))."""
+    _check_input(w, "w")
+    n, k = w.shape
+    nb = (n + 127) // 128
+    b_store = torch.empty(k, n, dtype=torch.float8_e4m3fn, device=w.device)
+    s_store = torch.empty(k // 128, nb, dtype=torch.float32, device=w.device)
+    with torch.cuda.device(w.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _lib.check(_lib.load().fp8bs_quantize_b(
+            w.data_ptr(), _DTYPES[w.dtype], w.stride(0) if n > 1 else max(k, 1),
+            b_store.data_ptr(), s_store.data_ptr(), n, k, stream))
+    return b_store.t(), s_store.t()

@@ -101,6 +101,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--configs", type=str, default="3,4,5", help="extra configurations reported under per_config")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-quant", dest="quant", action="store_false", help="skip the quantiser kernels under per_config")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run plain device copies of a known size (128 MiB read + 128 MiB written per copy), "
                          "the yardstick for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
@@ -186,6 +187,22 @@ def main():
             "name": cfg.name, "us": round(us, 2), "us_min": round(us_min, 2), "tflops": round(tf, 1), "gbs": round(gbs, 1),
             "input_sets": 1 if cfg.experts else nsets, "bound": bound, "frac": round(tf / PEAK_FP8_TFLOPS if bound == "mfma" else gbs / PEAK_HBM_GBS, 4)}
         d = sets = None
+    # ---- the quantisers in front of the GEMM (HBM-bound): activations of configuration 3, one expert's
+    # weights of configuration 5; 4 rotating inputs (> 256 MB in total) so that reads come from HBM ----
+    if args.quant:
+        quant = importlib.import_module("amd-developer-challenge-2025_amd.quant")
+        torch.cuda.empty_cache()
+        for name, rows, k, dt, fn in (("quant_a_fp32_4096x7168", 4096, 7168, torch.float32, quant.quantize_a),
+                                      ("quant_a_bf16_4096x7168", 4096, 7168, torch.bfloat16, quant.quantize_a),
+                                      ("quant_b_fp32_4096x7168", 4096, 7168, torch.float32, quant.quantize_b)):
+            g = torch.Generator(device=dev).manual_seed(1)
+            xs = [torch.randn(rows, k, generator=g, device=dev).to(dt) for _ in range(4 if dt == torch.float32 else 8)]
+            us, us_min = time_calls(lambda i: fn(xs[i % len(xs)]), args.steps, args.warmup)
+            nscale = rows * (k // 128) if fn is quant.quantize_a else ((rows + 127) // 128) * (k // 128)
+            by = rows * k * (xs[0].element_size() + 1) + 4 * nscale
+            per_config[name] = {"us": round(us, 2), "us_min": round(us_min, 2), "gbs": round(by / us * 1e-3, 1), "bytes": by,
+                                "input_sets": len(xs), "bound": "hbm", "frac": round(by / us * 1e-3 / PEAK_HBM_GBS, 4)}
+            xs = None
     result["per_config"] = per_config
 
     # ---- CPU baseline: the oracle on the same configuration-2 inputs, host cores ----

@@ -105,6 +105,28 @@ int fp8bs_gemm_grouped(const void* a, const void* b, const float* a_scale, const
                        void* c, const int32_t* row_offsets, int num_experts, int total_rows,
                        int n, int k, void* stream);
 
+/* ---- Quantisers (the step in front of the GEMM) -------------------------------------------------
+ * The reference has no counterpart: its operands arrive already quantised from the harness
+ * (1-amd-fp8-mm/0-amd-fp8-mm-new-begins.py:66-77).  These produce exactly those operands, in the
+ * storage layouts above, from a row-major fp32 or bf16 matrix.  Rule per block, bit for bit:
+ *   scale = max(max|x| / 448, 1e-12) (fp32),  q = e4m3fn(round to nearest even) of clamp(x / scale, +-448).
+ * `ldx` is the distance between input rows in elements (>= k; rows must start 16-byte aligned for
+ * fp32, 8-byte for bf16). */
+enum { FP8BS_DTYPE_F32 = 0, FP8BS_DTYPE_BF16 = 1 };
+
+/* Activations: x [m or src_rows][k] -> a (K rows of m bytes) and a_scale (K/128 rows of m floats), one
+ * scale per row and 128-wide K block.  If row_map is not NULL (device pointer, m int32 entries), output
+ * row i is quantised from input row row_map[i] (0 <= row_map[i] < src_rows; out-of-range entries give
+ * zero rows): the expert-contiguous gather of MoE tokens
+ * (2-amd-moe/3-amd-fp8-moe-hip-myhgemm.py:174-191) fused into the quantiser. */
+int fp8bs_quantize_a(const void* x, int x_dtype, int64_t ldx, const int32_t* row_map, int src_rows,
+                     void* a, float* a_scale, int m, int k, void* stream);
+
+/* Weights: w [n][k] -> b (K rows of n bytes) and b_scale (K/128 rows of ceil(n/128) floats), one scale
+ * per 128x128 block; a partial last block of rows takes its maximum over the rows that exist. */
+int fp8bs_quantize_b(const void* w, int w_dtype, int64_t ldw, void* b, float* b_scale, int n, int k,
+                     void* stream);
+
 #ifdef __cplusplus
 }
 #endif
