@@ -11,6 +11,7 @@ Layout of the package:
   submission.py   custom_kernel(data) / grouped_kernel(data): the reference's Python entry points
   inputs.py       host-side e4m3fn block quantisers and the synthetic inputs of the benchmark configurations
   quant.py        quantize_a / quantize_b: the HIP quantisers (fp32/bf16 -> operands in the GEMM's layout)
+  moe.py          topk / route: expert selection, row_offsets and the expert-contiguous row order
 """
 from .submission import custom_kernel, grouped_kernel, plan, workspace_bytes  # noqa: F401
 from . import inputs  # noqa: F401

@@ -14,6 +14,7 @@ EXPORTS = (
     "fp8bs_version", "fp8bs_strerror", "fp8bs_plan", "fp8bs_workspace_bytes",
     "fp8bs_gemm", "fp8bs_gemm_ex", "fp8bs_gemm_grouped",
     "fp8bs_quantize_a", "fp8bs_quantize_b",
+    "fp8bs_moe_topk", "fp8bs_moe_route_workspace_bytes", "fp8bs_moe_route",
 )
 
 VARIANT_NAMES = {0: "auto", 1: "generic", 2: "t256x256", 3: "t128x128", 4: "t64x128", 5: "t256x128", 6: "skinny64x144"}
@@ -62,6 +63,12 @@ def load() -> ctypes.CDLL:
     lib.fp8bs_quantize_a.argtypes = [vp, i32, i64, vp, i32, vp, vp, i32, i32, vp]
     lib.fp8bs_quantize_b.restype = i32
     lib.fp8bs_quantize_b.argtypes = [vp, i32, i64, vp, vp, i32, i32, vp]
+    lib.fp8bs_moe_topk.restype = i32
+    lib.fp8bs_moe_topk.argtypes = [vp, i32, i32, i32, vp, vp]
+    lib.fp8bs_moe_route_workspace_bytes.restype = sz
+    lib.fp8bs_moe_route_workspace_bytes.argtypes = [i32, i32]
+    lib.fp8bs_moe_route.restype = i32
+    lib.fp8bs_moe_route.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, sz, vp]
     _lib = lib
     return lib
 

@@ -11,7 +11,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 LIB_PATH = os.path.join(HERE, "libfp8bs.so")
-SOURCES = [os.path.join(HERE, "csrc", f) for f in ("fp8bs_kernels.hip", "fp8bs_api.hip", "fp8bs_quant.hip")]
+SOURCES = [os.path.join(HERE, "csrc", f) for f in ("fp8bs_kernels.hip", "fp8bs_api.hip", "fp8bs_quant.hip", "fp8bs_route.hip")]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++20", "-shared", "-fPIC",

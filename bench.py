@@ -203,6 +203,24 @@ def main():
             per_config[name] = {"us": round(us, 2), "us_min": round(us_min, 2), "gbs": round(by / us * 1e-3, 1), "bytes": by,
                                 "input_sets": len(xs), "bound": "hbm", "frac": round(by / us * 1e-3 / PEAK_HBM_GBS, 4)}
             xs = None
+        # routing of configuration 5 (4096 tokens, 32 experts, top 8): launch-bound bookkeeping, then the
+        # quantiser gathering 32768 expert-contiguous rows out of the 4096 token rows
+        moe = importlib.import_module("amd-developer-challenge-2025_amd.moe")
+        cfg5 = pkg.inputs.CONFIGS[4]
+        g = torch.Generator(device=dev).manual_seed(cfg5.seed)
+        scores = torch.rand(cfg5.m, cfg5.experts, generator=g, device=dev)
+        us, us_min = time_calls(lambda i: moe.route(moe.topk(scores, cfg5.topk), cfg5.experts), args.steps, args.warmup)
+        per_config["moe_topk_route_4096x32_top8"] = {"us": round(us, 2), "us_min": round(us_min, 2), "bound": "launch",
+                                                     "kernels": 3, "note": "top-k + count + assign (scan fused), no host sync; mostly the Python wrapper's allocations"}
+        row_map = moe.route(moe.topk(scores, cfg5.topk), cfg5.experts)[1]
+        x = torch.randn(cfg5.m, cfg5.k, generator=g, device=dev)
+        us, us_min = time_calls(lambda i: quant.quantize_a(x, row_map), max(args.steps // 2, 5), 3)
+        rows = row_map.numel()
+        by = cfg5.m * cfg5.k * 4 + rows * cfg5.k + 4 * rows * (cfg5.k // 128)
+        per_config["quant_a_gather_fp32_4096to32768x7168"] = {
+            "us": round(us, 2), "us_min": round(us_min, 2), "gbs": round(by / us * 1e-3, 1), "bytes": by, "bound": "hbm",
+            "frac": round(by / us * 1e-3 / PEAK_HBM_GBS, 4), "note": "token rows read once algorithmically, written 8 times"}
+        x = row_map = scores = None
     result["per_config"] = per_config
 
     # ---- CPU baseline: the oracle on the same configuration-2 inputs, host cores ----

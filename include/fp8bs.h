@@ -127,6 +127,29 @@ int fp8bs_quantize_a(const void* x, int x_dtype, int64_t ldx, const int32_t* row
 int fp8bs_quantize_b(const void* w, int w_dtype, int64_t ldw, void* b, float* b_scale, int n, int k,
                      void* stream);
 
+/* ---- MoE routing (the caller of the grouped GEMM) ------------------------------------------------
+ * Top-k selection with the reference's rule (2-amd-moe/amd-moe-submission.py:32-56, 58-105): per token,
+ * k times the strictly greatest score not yet taken, lowest index first among equals, best first; NaN
+ * and -inf are never selected (index -1, as in the reference).  scores: [tokens][experts] fp32
+ * row-major; top_idx: [tokens][topk] int32. */
+int fp8bs_moe_topk(const float* scores, int tokens, int experts, int topk, int32_t* top_idx, void* stream);
+
+/* Bytes of device workspace fp8bs_moe_route needs. */
+size_t fp8bs_moe_route_workspace_bytes(int tokens, int experts);
+
+/* From top_idx [tokens][topk] (entries outside [0, experts) are ignored) build, on the device and with
+ * no host synchronisation (the reference synchronises and reads the counts on the host, :230-234):
+ *   row_offsets [experts+1]   exclusive prefix of the rows per expert, total appended
+ *                              (2-amd-moe/3-amd-fp8-moe-hip-myhgemm.py:142-148) - what fp8bs_gemm_grouped takes
+ *   row_map     [tokens*topk] row_map[row] = token that fills that row; rows of an expert are ordered by
+ *                              token id (the reference hands positions out by atomicAdd, :107-156, so its
+ *                              order varies between runs) - what fp8bs_quantize_a takes as its gather list;
+ *                              entries beyond row_offsets[experts] are not written
+ *   slot_of     [tokens][topk] row of every (token, choice), -1 for ignored entries; may be NULL
+ * experts <= 1024, topk <= 16. */
+int fp8bs_moe_route(const int32_t* top_idx, int tokens, int experts, int topk, int32_t* row_offsets,
+                    int32_t* row_map, int32_t* slot_of, void* ws, size_t ws_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
