@@ -214,4 +214,23 @@ int fp8bs_gemm_grouped(const void* a, const void* b, const float* a_scale, const
     return FP8BS_OK;
 }
 
+int fp8bs_gemm_silu_mul(const void* a, const void* b, const float* a_scale, const float* b_scale, void* h,
+                        const int32_t* row_offsets, int num_experts, int rows, int n, int k, void* stream) {
+    if (row_offsets && num_experts <= 0) return FP8BS_ERR_BAD_OFFSETS;
+    if ((n & 1) != 0) return FP8BS_ERR_BAD_SHAPE;
+    int st = check_common(a, b, a_scale, b_scale, h, rows, n, k);
+    if (st != FP8BS_OK) return st;
+    if (rows == 0 || n == 0) return FP8BS_OK;
+    fp8bs::GemmArgs g{};
+    g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.as = a_scale; g.bs = b_scale;
+    g.c = (uint16_t*)h; g.ws = nullptr; g.row_offsets = row_offsets;
+    g.m = rows; g.n = n; g.k = k; g.lda = rows; g.nb = (n + 127) / 128;
+    g.split_k = 1; g.kb_per_split = k / KBLK; g.band_h = 4; g.num_experts = row_offsets ? num_experts : 0;
+    g.epi = 1;
+    // 16-byte stores of n/2-wide bf16 rows need n % 16 == 0 as the copies do
+    int variant = (k == 0 || (rows % 16) != 0 || (n % 16) != 0) ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
+    if (fp8bs::launch_gemm(variant, row_offsets ? 2 : 0, g, (hipStream_t)stream) != hipSuccess) return FP8BS_ERR_LAUNCH;
+    return FP8BS_OK;
+}
+
 }  // extern "C"

@@ -22,6 +22,7 @@ struct GemmArgs {
     int split_k, kb_per_split;
     int band_h;             // tile rows per band of the tile walk
     int num_experts;
+    int epi;                // 0: bf16 of the product; 1: silu(column 2i) * column 2i+1, n/2 output columns
 };
 
 // mode: 0 dense bf16, 1 dense split-K partials, 2 grouped.  variant: FP8BS_VARIANT_* (not AUTO).

@@ -122,7 +122,16 @@ __device__ __forceinline__ int swz_of_krow(int krow) {
     return (krow / (16 / CPR)) % CPR;
 }
 
-template <int BM, int BN, int WM, int WN, int MODE>
+// EPI 0: plain bf16 output.  EPI 1: gate/up pairs - column 2i is gate_i, column 2i+1 is up_i - are
+// combined to silu(gate_i) * up_i in fp32 and the output has n/2 columns (role of the fp16 layer's
+// re_silu_mul_kernel, 2-amd-moe/amd-moe-submission.py:366-407, fused into the GEMM as in
+// 2-amd-moe/5-amd-fp8-moe-hip-fuse.py:366-408).
+__device__ __forceinline__ float silu_mul(float gate, float up) {
+    // gate / (1 + exp(-gate)) * up; exp2 and rcp are the hardware approximations (~1 ulp)
+    return gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * gate)) * up;
+}
+
+template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64)
 void gemm_tr_kernel(const GemmArgs p) {
     using C = TileCfg<BM, BN, WM, WN, MODE>;
@@ -389,32 +398,40 @@ void gemm_tr_kernel(const GemmArgs p) {
         // free: after the barrier of the last K block no wave reads them and no copy is in flight.
         // Each wave uses its own WM x WN bf16 region; 16-byte chunks are XOR-swizzled by row so that
         // neither the 8-byte writes (16 rows per instruction) nor the 16-byte reads conflict.
-        constexpr int ROW_CHUNKS = WN * 2 / 16;                       // 16-byte chunks per tile row
+        constexpr int WNO = EPI == 1 ? WN / 2 : WN;                   // output columns of the wave tile
+        constexpr int ROW_CHUNKS = WNO * 2 / 16;                      // 16-byte chunks per tile row
         constexpr int ROWS_PER_SWEEP = 16 / ROW_CHUNKS > 0 ? 16 / ROW_CHUNKS : 1;
-        unsigned char* region = lds + wave * (WM * WN * 2);
+        unsigned char* region = lds + wave * (WM * WNO * 2);
 #pragma unroll
         for (int t = 0; t < C::MT; t++) {
             const int r = 16 * t + i16;
             const int sw = (r / ROWS_PER_SWEEP) % ROW_CHUNKS;
 #pragma unroll
             for (int u = 0; u < C::NT; u++) {
-                v2i o;
-                o[0] = (int)pack_bf16x2(acc[t][u][0], acc[t][u][1]);
-                o[1] = (int)pack_bf16x2(acc[t][u][2], acc[t][u][3]);
-                const int chunk = 2 * u + (g >> 1);
-                *(v2i*)(region + r * (WN * 2) + ((chunk ^ sw) << 4) + (g & 1) * 8) = o;
+                if (EPI == 1) {
+                    // the lane's four columns are two (gate, up) pairs -> two outputs, 4 bytes
+                    const uint32_t o = pack_bf16x2(silu_mul(acc[t][u][0], acc[t][u][1]), silu_mul(acc[t][u][2], acc[t][u][3]));
+                    *(uint32_t*)(region + r * (WNO * 2) + ((u ^ sw) << 4) + g * 4) = o;
+                } else {
+                    v2i o;
+                    o[0] = (int)pack_bf16x2(acc[t][u][0], acc[t][u][1]);
+                    o[1] = (int)pack_bf16x2(acc[t][u][2], acc[t][u][3]);
+                    const int chunk = 2 * u + (g >> 1);
+                    *(v2i*)(region + r * (WNO * 2) + ((chunk ^ sw) << 4) + (g & 1) * 8) = o;
+                }
             }
         }
         constexpr int PASSES = WM * ROW_CHUNKS / 64;
+        const int ldc = EPI == 1 ? p.n / 2 : p.n;
 #pragma unroll
         for (int q = 0; q < PASSES; q++) {
             const int idx = q * 64 + lane;
             const int r = idx / ROW_CHUNKS, chunk = idx % ROW_CHUNKS;
             const int sw = (r / ROWS_PER_SWEEP) % ROW_CHUNKS;
-            const v4i val = *(const v4i*)(region + r * (WN * 2) + ((chunk ^ sw) << 4));
-            const int row = m0 + wave_m * WM + r, col = n0 + wave_n * WN + chunk * 8;
-            if (row >= row_lo && row < row_hi && col < p.n)
-                *(v4i*)(p.c + (size_t)row * p.n + col) = val;
+            const v4i val = *(const v4i*)(region + r * (WNO * 2) + ((chunk ^ sw) << 4));
+            const int row = m0 + wave_m * WM + r, col = (EPI == 1 ? (n0 + wave_n * WN) / 2 : n0 + wave_n * WN) + chunk * 8;
+            if (row >= row_lo && row < row_hi && col < ldc)
+                *(v4i*)(p.c + (size_t)row * ldc + col) = val;
         }
     }
 }
@@ -638,11 +655,23 @@ __device__ __forceinline__ float e4m3fn_to_float(uint32_t v) {
     return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, f) | s);
 }
 
+__device__ __forceinline__ float generic_dot(const GemmArgs& p, const uint8_t* b, const float* bs, int row, int col) {
+    float accum = 0.f;
+    for (int kb = 0; kb < p.k / KBLK; kb++) {
+        float part = 0.f;
+        for (int kk = kb * KBLK; kk < (kb + 1) * KBLK; kk++)
+            part = __builtin_fmaf(e4m3fn_to_float(p.a[(size_t)kk * p.lda + row]), e4m3fn_to_float(b[(size_t)kk * p.n + col]), part);
+        accum = __builtin_fmaf(part, p.as[(size_t)kb * p.lda + row] * bs[(size_t)kb * p.nb + col / 128], accum);
+    }
+    return accum;
+}
+
 __global__ __launch_bounds__(256)
 void gemm_generic_kernel(const GemmArgs p) {
-    int col = blockIdx.x * 16 + (threadIdx.x & 15);
+    int col = blockIdx.x * 16 + (threadIdx.x & 15);            // output column (epi 1: pair index)
     int row = blockIdx.y * 16 + (threadIdx.x >> 4);
-    if (row >= p.m || col >= p.n) return;
+    const int ncols = p.epi == 1 ? p.n / 2 : p.n;
+    if (row >= p.m || col >= ncols) return;
     const uint8_t* b = p.b;
     const float* bs = p.bs;
     if (p.row_offsets) {
@@ -651,25 +680,25 @@ void gemm_generic_kernel(const GemmArgs p) {
         b += (size_t)e * p.k * p.n;
         bs += (size_t)e * (p.k / KBLK) * p.nb;
     }
-    float accum = 0.f;
-    for (int kb = 0; kb < p.k / KBLK; kb++) {
-        float part = 0.f;
-        for (int kk = kb * KBLK; kk < (kb + 1) * KBLK; kk++)
-            part = __builtin_fmaf(e4m3fn_to_float(p.a[(size_t)kk * p.lda + row]), e4m3fn_to_float(b[(size_t)kk * p.n + col]), part);
-        accum = __builtin_fmaf(part, p.as[(size_t)kb * p.lda + row] * bs[(size_t)kb * p.nb + col / 128], accum);
+    float accum;
+    if (p.epi == 1) {
+        const float gate = generic_dot(p, b, bs, row, 2 * col), up = generic_dot(p, b, bs, row, 2 * col + 1);
+        accum = gate / (1.0f + __expf(-gate)) * up;
+    } else {
+        accum = generic_dot(p, b, bs, row, col);
     }
     v2f f = {accum, 0.f};
     v2bf h = __builtin_convertvector(f, v2bf);
-    p.c[(size_t)row * p.n + col] = __builtin_bit_cast(uint32_t, h) & 0xFFFFu;
+    p.c[(size_t)row * ncols + col] = __builtin_bit_cast(uint32_t, h) & 0xFFFFu;
 }
 
 // ---------------------------------------------------------------------------------------------------
 // Launchers
 // ---------------------------------------------------------------------------------------------------
-template <int BM, int BN, int WM, int WN, int MODE>
+template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0>
 static hipError_t launch_tr(const GemmArgs& a, dim3 grid, hipStream_t stream) {
     using C = TileCfg<BM, BN, WM, WN, MODE>;
-    auto kern = gemm_tr_kernel<BM, BN, WM, WN, MODE>;
+    auto kern = gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI>;
     static bool attr_done = false;   // raising the dynamic-LDS limit is idempotent; a race is harmless
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
@@ -680,8 +709,22 @@ static hipError_t launch_tr(const GemmArgs& a, dim3 grid, hipStream_t stream) {
     return hipGetLastError();
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, bool WITH_EPI = false>
 static hipError_t launch_shape(const GemmArgs& a, int mode, hipStream_t stream) {
+    if (a.epi != 0) {
+        // the fused silu-mul epilogue exists for the 256x256 tile, dense or grouped, without K split
+        if constexpr (WITH_EPI) {
+            int tiles_n = (a.n + BN - 1) / BN;
+            if (a.epi != 1 || mode == 1) return hipErrorInvalidValue;
+            if (mode == 2) {
+                long slots = ((long)a.m + BM - 1) / BM + 2L * a.num_experts;
+                return launch_tr<BM, BN, WM, WN, 2, 1>(a, dim3(tiles_n, (unsigned)slots), stream);
+            }
+            return launch_tr<BM, BN, WM, WN, 0, 1>(a, dim3(((a.m + BM - 1) / BM) * tiles_n), stream);
+        } else {
+            return hipErrorInvalidValue;
+        }
+    }
     if (mode == 2) {
         int tiles_n = (a.n + BN - 1) / BN;
         // upper bound on m-tile slots: every expert can waste up to 15 rows (aligned-down start)
@@ -697,11 +740,11 @@ static hipError_t launch_shape(const GemmArgs& a, int mode, hipStream_t stream) 
 hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t stream) {
     switch (variant) {
         case 1: {
-            dim3 grid((a.n + 15) / 16, (a.m + 15) / 16);
+            dim3 grid(((a.epi == 1 ? a.n / 2 : a.n) + 15) / 16, (a.m + 15) / 16);
             hipLaunchKernelGGL(gemm_generic_kernel, grid, dim3(256), 0, stream, a);
             return hipGetLastError();
         }
-        case 2: return launch_shape<256, 256, 64, 128>(a, mode, stream);
+        case 2: return launch_shape<256, 256, 64, 128, true>(a, mode, stream);
         case 3: return launch_shape<128, 128, 64, 64>(a, mode, stream);
         case 4: return launch_shape<64, 128, 32, 64>(a, mode, stream);
         case 5: return launch_shape<256, 128, 64, 64>(a, mode, stream);

@@ -221,6 +221,39 @@ void route_assign_kernel(const int32_t* __restrict__ top_idx, int tokens, int ex
     }
 }
 
+// out[t][d] = sum_j weights[t][j] * y[slot_of[t][j]][d], fp32 accumulation in the order j = 0..topk-1,
+// one rounding to bf16 (role of pack_output, 2-amd-moe/amd-moe-submission.py:239-301, which accumulates
+// in fp16).  One block per token, 8 columns (16 bytes) per thread and step; entries with slot -1 are skipped.
+typedef int cv4i __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(RB)
+void moe_combine_kernel(const uint16_t* __restrict__ y, const int32_t* __restrict__ slot_of, const float* __restrict__ weights,
+                        uint16_t* __restrict__ out, int topk, int d) {
+    const int t = blockIdx.x;
+    for (int c = threadIdx.x * 8; c < d; c += RB * 8) {
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < topk; j++) {
+            const int slot = slot_of[(size_t)t * topk + j];
+            if (slot < 0) continue;
+            const float w = weights[(size_t)t * topk + j];
+            const cv4i v = *(const cv4i*)(y + (size_t)slot * d + c);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                acc[2 * i] = __builtin_fmaf(w, __builtin_bit_cast(float, (uint32_t)v[i] << 16), acc[2 * i]);
+                acc[2 * i + 1] = __builtin_fmaf(w, __builtin_bit_cast(float, (uint32_t)v[i] & 0xFFFF0000u), acc[2 * i + 1]);
+            }
+        }
+        cv4i o;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            typedef float cv2f __attribute__((ext_vector_type(2)));
+            typedef __bf16 cv2bf __attribute__((ext_vector_type(2)));
+            cv2f f = {acc[2 * i], acc[2 * i + 1]};
+            o[i] = (int)__builtin_bit_cast(uint32_t, __builtin_convertvector(f, cv2bf));
+        }
+        *(cv4i*)(out + (size_t)t * d + c) = o;
+    }
+}
+
 }  // namespace fp8bs
 
 extern "C" int fp8bs_moe_topk(const float* scores, int tokens, int experts, int topk, int32_t* top_idx, void* stream) {
@@ -265,5 +298,15 @@ extern "C" int fp8bs_moe_route(const int32_t* top_idx, int tokens, int experts, 
         hipLaunchKernelGGL(fp8bs::route_assign_kernel<false>, dim3(nblocks), dim3(fp8bs::RB), 0, s, top_idx, tokens, experts, topk,
                            (const int32_t*)ws, row_offsets, row_map, slot_of);
     }
+    return hipGetLastError() == hipSuccess ? FP8BS_OK : FP8BS_ERR_LAUNCH;
+}
+
+extern "C" int fp8bs_moe_combine(const void* y, const int32_t* slot_of, const float* weights, void* out,
+                                 int tokens, int topk, int d, void* stream) {
+    if (tokens < 0 || topk <= 0 || d < 0 || (d % 8) != 0) return FP8BS_ERR_BAD_SHAPE;
+    if (tokens == 0 || d == 0) return FP8BS_OK;
+    if (!y || !slot_of || !weights || !out) return FP8BS_ERR_NULL_POINTER;
+    hipLaunchKernelGGL(fp8bs::moe_combine_kernel, dim3(tokens), dim3(fp8bs::RB), 0, (hipStream_t)stream,
+                       (const uint16_t*)y, slot_of, weights, (uint16_t*)out, topk, d);
     return hipGetLastError() == hipSuccess ? FP8BS_OK : FP8BS_ERR_LAUNCH;
 }

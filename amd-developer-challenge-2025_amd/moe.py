@@ -46,3 +46,56 @@ def route(top_idx: torch.Tensor, experts: int) -> Tuple[torch.Tensor, torch.Tens
         _lib.check(lib.fp8bs_moe_route(top_idx.data_ptr(), t, experts, k, row_offsets.data_ptr(), row_map.data_ptr(),
                                        slot_of.data_ptr(), ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream))
     return row_offsets, row_map, slot_of
+
+
+def gate_up_silu(data):
+    """Gate/up projection with silu(gate) * up fused into the GEMM: ``data = (a, b, a_scale, b_scale, row_offsets, h)``.
+
+    ``b`` holds gate and up weights interleaved by row (row 2i = gate_i, row 2i+1 = up_i), [E, n, k] with
+    every expert K-major (or [n, k] K-major with ``row_offsets=None`` for one dense weight); ``h`` is
+    bf16 [rows, n/2].  Role of re_silu_mul_kernel (2-amd-moe/amd-moe-submission.py:366-407) fused as in
+    2-amd-moe/5-amd-fp8-moe-hip-fuse.py:366-408.  Fills and returns ``h``.
+    """
+    a, b, a_scale, b_scale, row_offsets, h = data
+    rows, k = a.shape
+    grouped = row_offsets is not None
+    num_experts = b.shape[0] if grouped else 0
+    n = b.shape[1] if grouped else b.shape[0]
+    if a.dtype != torch.float8_e4m3fn or b.dtype != torch.float8_e4m3fn or a_scale.dtype != torch.float32 \
+            or b_scale.dtype != torch.float32 or h.dtype != torch.bfloat16:
+        raise TypeError("a, b must be float8_e4m3fn, the scales float32, h bfloat16")
+    if n % 2 or tuple(h.shape) != (rows, n // 2) or not h.is_contiguous():
+        raise ValueError("h must be a contiguous [rows, n/2] tensor")
+    if k % 128 or not a.t().is_contiguous() or not a_scale.t().is_contiguous():
+        raise ValueError("a / a_scale must be K-major with k a multiple of 128")
+    bt = b.transpose(1, 2) if grouped else b.t()
+    bst = b_scale.transpose(1, 2) if grouped else b_scale.t()
+    if not bt.is_contiguous() or not bst.is_contiguous():
+        raise ValueError("b and b_scale must be K-major (per expert)")
+    if grouped and (row_offsets.dtype != torch.int32 or tuple(row_offsets.shape) != (num_experts + 1,) or not row_offsets.is_cuda):
+        raise ValueError("row_offsets must be an int32 GPU tensor with num_experts+1 entries")
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.load().fp8bs_gemm_silu_mul(
+            a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(), h.data_ptr(),
+            row_offsets.data_ptr() if grouped else None, num_experts, rows, n, k,
+            torch.cuda.current_stream().cuda_stream))
+    return h
+
+
+def combine(y: torch.Tensor, slot_of: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
+    """out[t] = sum_j weights[t, j] * y[slot_of[t, j]]  (y bf16 [rows, d], weights fp32 [T, k]) -> bf16 [T, d].
+
+    Role of pack_output (2-amd-moe/amd-moe-submission.py:239-301); fp32 accumulation in the order of j.
+    """
+    if y.dtype != torch.bfloat16 or y.dim() != 2 or not y.is_contiguous() or not y.is_cuda:
+        raise ValueError("y must be a contiguous bfloat16 [rows, d] tensor on the GPU")
+    if slot_of.dtype != torch.int32 or not slot_of.is_contiguous() or weights.dtype != torch.float32 \
+            or not weights.is_contiguous() or slot_of.shape != weights.shape or slot_of.dim() != 2:
+        raise ValueError("slot_of (int32) and weights (float32) must be contiguous [tokens, topk] tensors")
+    t, k = slot_of.shape
+    d = y.shape[1]
+    out = torch.empty(t, d, dtype=torch.bfloat16, device=y.device)
+    with torch.cuda.device(y.device):
+        _lib.check(_lib.load().fp8bs_moe_combine(y.data_ptr(), slot_of.data_ptr(), weights.data_ptr(), out.data_ptr(),
+                                                 t, k, d, torch.cuda.current_stream().cuda_stream))
+    return out

@@ -221,6 +221,45 @@ def main():
             "us": round(us, 2), "us_min": round(us_min, 2), "gbs": round(by / us * 1e-3, 1), "bytes": by, "bound": "hbm",
             "frac": round(by / us * 1e-3 / PEAK_HBM_GBS, 4), "note": "token rows read once algorithmically, written 8 times"}
         x = row_map = scores = None
+        # expert FFN of configuration 5: gate/up GEMM with the fused silu-mul epilogue (N = 2 x 2048
+        # interleaved), quantisation of h, down projection (N = 7168, K = 2048), weighted un-permute
+        torch.cuda.empty_cache()
+        d5 = gpu_grouped_inputs(pkg, cfg5, dev, cfg5.seed)
+        a5, b5, as5, bs5, ro5, _ = d5
+        rows = a5.shape[0]
+        h = torch.empty(rows, cfg5.n // 2, dtype=torch.bfloat16, device=dev)
+        us, us_min = time_calls(lambda i: moe.gate_up_silu((a5, b5, as5, bs5, ro5, h)), max(args.steps // 5, 5), 3)
+        fl = 2.0 * rows * cfg5.n * cfg5.k
+        per_config["ffn_gate_up_silu_32768x4096x7168"] = {"us": round(us, 2), "us_min": round(us_min, 2), "tflops": round(fl / us * 1e-6, 1),
+                                                          "bound": "mfma", "frac": round(fl / us * 1e-6 / PEAK_FP8_TFLOPS, 4)}
+        d5 = a5 = b5 = as5 = bs5 = None
+        torch.cuda.empty_cache()
+        di = cfg5.n // 2
+        us, us_min = time_calls(lambda i: quant.quantize_a(h), max(args.steps // 2, 5), 3)
+        by = rows * di * 3 + 4 * rows * (di // 128)
+        per_config["quant_a_bf16_32768x2048"] = {"us": round(us, 2), "us_min": round(us_min, 2), "gbs": round(by / us * 1e-3, 1), "bytes": by,
+                                                 "bound": "hbm", "frac": round(by / us * 1e-3 / PEAK_HBM_GBS, 4)}
+        a2, a2s = quant.quantize_a(h)
+        g = torch.Generator(device=dev).manual_seed(7)
+        b2 = torch.empty(cfg5.experts, di, cfg5.k, dtype=torch.float8_e4m3fn, device=dev)           # storage [E][K=di][N=7168]
+        b2s = torch.empty(cfg5.experts, di // 128, cfg5.k // 128, dtype=torch.float32, device=dev)
+        for e in range(cfg5.experts):
+            qb, sb = quant.quantize_b(torch.randn(cfg5.k, di, generator=g, device=dev) * 0.02)
+            b2[e], b2s[e] = qb.t(), sb.t()
+        y = torch.empty(rows, cfg5.k, dtype=torch.bfloat16, device=dev)
+        dd = (a2, b2.transpose(1, 2), a2s, b2s.transpose(1, 2), ro5, y)
+        us, us_min = time_calls(lambda i: pkg.grouped_kernel(dd), max(args.steps // 5, 5), 3)
+        fl = 2.0 * rows * cfg5.k * di
+        per_config["ffn_down_32768x7168x2048"] = {"us": round(us, 2), "us_min": round(us_min, 2), "tflops": round(fl / us * 1e-6, 1),
+                                                  "bound": "mfma", "frac": round(fl / us * 1e-6 / PEAK_FP8_TFLOPS, 4)}
+        slot = torch.randperm(rows, device=dev).reshape(cfg5.m, cfg5.topk).to(torch.int32)
+        wts = torch.rand(cfg5.m, cfg5.topk, device=dev)
+        us, us_min = time_calls(lambda i: moe.combine(y, slot, wts), max(args.steps // 2, 5), 3)
+        by = rows * cfg5.k * 2 + cfg5.m * cfg5.k * 2 + rows * 8
+        per_config["moe_combine_4096x8x7168"] = {"us": round(us, 2), "us_min": round(us_min, 2), "gbs": round(by / us * 1e-3, 1), "bytes": by,
+                                                 "bound": "hbm", "frac": round(by / us * 1e-3 / PEAK_HBM_GBS, 4),
+                                                 "note": "y (470 MB) was just written and may partly sit in the 256 MB cache"}
+        dd = a2 = b2 = y = h = None
     result["per_config"] = per_config
 
     # ---- CPU baseline: the oracle on the same configuration-2 inputs, host cores ----

@@ -150,6 +150,22 @@ size_t fp8bs_moe_route_workspace_bytes(int tokens, int experts);
 int fp8bs_moe_route(const int32_t* top_idx, int tokens, int experts, int topk, int32_t* row_offsets,
                     int32_t* row_map, int32_t* slot_of, void* ws, size_t ws_bytes, void* stream);
 
+/* ---- Expert FFN pieces behind the grouped GEMM ---------------------------------------------------
+ * Gate/up projection with the activation fused into the GEMM's epilogue.  b holds the gate and up
+ * weights interleaved by row: row 2i = gate_i, row 2i+1 = up_i (n = 2 x intermediate size, even);
+ * h[row][i] = bf16( silu(C[row][2i]) * C[row][2i+1] ) with C the fp32 block-scaled product, h has n/2
+ * columns.  Role of re_silu_mul_kernel (2-amd-moe/amd-moe-submission.py:366-407; fp16 there, rounding
+ * silu to fp16 before the product) fused as in 2-amd-moe/5-amd-fp8-moe-hip-fuse.py:366-408.
+ * row_offsets NULL: dense (one weight matrix); else grouped as fp8bs_gemm_grouped. */
+int fp8bs_gemm_silu_mul(const void* a, const void* b, const float* a_scale, const float* b_scale, void* h,
+                        const int32_t* row_offsets, int num_experts, int rows, int n, int k, void* stream);
+
+/* Weighted un-permute: out[t][:] = sum_j weights[t][j] * y[slot_of[t][j]][:]  (y, out bf16 with d columns,
+ * d % 8 == 0; fp32 accumulation in the order j = 0..topk-1, one rounding; slot -1 is skipped).  Role of
+ * pack_output (2-amd-moe/amd-moe-submission.py:239-301; fp16 accumulation there). */
+int fp8bs_moe_combine(const void* y, const int32_t* slot_of, const float* weights, void* out,
+                      int tokens, int topk, int d, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
