@@ -113,7 +113,6 @@ struct TileCfg {
     static_assert(A_BYTES % (16 * NTHREADS) == 0 && B_BYTES % (16 * NTHREADS) == 0, "tile/threads");
     static_assert(WN <= 128 && 128 % WN == 0, "a wave's n range must stay inside one b_scale block");
     static_assert(CPR_A <= 16 && CPR_B <= 16, "swizzle assumes a k row spans at most 256 bytes");
-    static_assert(BM * BN * 2 <= LDS_BYTES, "the bf16 epilogue stages the whole tile in LDS");
 };
 
 template <int CPR>
@@ -143,87 +142,124 @@ void gemm_tr_kernel(const GemmArgs p) {
     const int g = lane >> 4, i16 = lane & 15;
     const int wave_m = wave % C::WAVES_M, wave_n = wave / C::WAVES_M;
 
-    // ---- which tile ---------------------------------------------------------------------------
-    int m0, n0, kb_begin, kb_end, split_z = 0;
-    int row_lo = 0, row_hi = p.m;                  // rows this workgroup may store
-    const uint8_t* bptr = p.b;
-    const float* bsptr = p.bs;
-    if (MODE == 2) {
-        // grouped: workgroup (blockIdx.x = tile_n, blockIdx.y = m-tile slot).  Slots are laid over
-        // the experts in order; expert e's tiles start at row_offsets[e] rounded down to 16 so that
-        // global 16-byte loads stay aligned; rows outside [row_offsets[e], row_offsets[e+1]) are
-        // computed but never stored.
-        int slot = blockIdx.y;
-        int e = 0, found = 0, start = 0, cnt_lo = 0, cnt_hi = 0;
-        int acc_tiles = 0;
+    // ---- tiles ---------------------------------------------------------------------------------
+    // The workgroup is persistent: it walks the tiles  blockIdx.x, blockIdx.x + gridDim.x, ...  and
+    // issues the first K block of the next tile before it converts and stores the current one, so a
+    // tile's output and the next tile's first loads overlap (with K = 2048 the per-tile prologue and
+    // epilogue are a third of a tile's time otherwise).
+    struct Tile {
+        int valid, m0, n0, kb_begin, kb_end, split_z, row_lo, row_hi;
+        const uint8_t* bptr;
+        const float* bsptr;
+    };
+    int total_slots = 0;                      // grouped: m-tile slots that exist (from row_offsets)
+    if (MODE == 2)
         for (int x = 0; x < p.num_experts; x++) {
-            int lo = p.row_offsets[x], hi = p.row_offsets[x + 1];
-            int s = lo & ~15;
-            int nt = (hi > lo) ? (hi - s + BM - 1) / BM : 0;
-            if (!found && slot < acc_tiles + nt) {
-                found = 1; e = x; start = s + (slot - acc_tiles) * BM; cnt_lo = lo; cnt_hi = hi;
-            }
-            acc_tiles += nt;
+            const int lo = p.row_offsets[x], hi = p.row_offsets[x + 1];
+            total_slots += (hi > lo) ? (hi - (lo & ~15) + BM - 1) / BM : 0;
         }
-        if (!found) return;                        // uniform for the whole workgroup
-        m0 = start; n0 = blockIdx.x * BN;
-        row_lo = cnt_lo; row_hi = cnt_hi;
-        bptr += (size_t)e * (size_t)p.k * (size_t)p.n;
-        bsptr += (size_t)e * (size_t)(p.k / KBLK) * (size_t)p.nb;
-        kb_begin = 0; kb_end = p.k / KBLK;
-    } else {
-        int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
-        int per_split = tiles_m * tiles_n;
-        int v = xcd_virtual_id(blockIdx.x, per_split * p.split_k);
-        split_z = v / per_split;
-        int tm, tn;
-        band_tile(v - split_z * per_split, tiles_m, tiles_n, p.band_h, tm, tn);
-        m0 = tm * BM; n0 = tn * BN;
-        int kbt = p.k / KBLK;
-        kb_begin = split_z * p.kb_per_split;
-        kb_end = kb_begin + p.kb_per_split;
-        kb_end = kb_end < kbt ? kb_end : kbt;
-    }
+    auto pick_tile = [&](int it) -> Tile {
+        Tile t;
+        t.valid = 0; t.m0 = 0; t.n0 = 0; t.kb_begin = 0; t.kb_end = 0; t.split_z = 0; t.row_lo = 0; t.row_hi = p.m;
+        t.bptr = p.b; t.bsptr = p.bs;
+        const int G = gridDim.x;
+        if (MODE == 2) {
+            // grouped: m-tile slots are laid over the experts in order; expert e's tiles start at
+            // row_offsets[e] rounded down to 16 so that global 16-byte loads stay aligned; rows outside
+            // [row_offsets[e], row_offsets[e+1]) are computed but never stored.  The gridDim.x tiles in
+            // flight together are dealt to the XCDs in contiguous runs and laid over the (slot, n tile)
+            // grid in bands of band_h slots, as in the dense case, so that the tiles sharing an L2 form a
+            // compact block of few A panels and few B panels.
+            const int tiles_n = (p.n + BN - 1) / BN;
+            const int total = total_slots * tiles_n;
+            const int v = it * G + xcd_virtual_id(blockIdx.x, G);
+            if (v >= total) return t;
+            int slot, tn;
+            band_tile(v, total_slots, tiles_n, p.band_h, slot, tn);
+            int e = 0, found = 0, start = 0, cnt_lo = 0, cnt_hi = 0;
+            int acc_tiles = 0;
+            for (int x = 0; x < p.num_experts; x++) {
+                int lo = p.row_offsets[x], hi = p.row_offsets[x + 1];
+                int s = lo & ~15;
+                int nt = (hi > lo) ? (hi - s + BM - 1) / BM : 0;
+                if (!found && slot < acc_tiles + nt) {
+                    found = 1; e = x; start = s + (slot - acc_tiles) * BM; cnt_lo = lo; cnt_hi = hi;
+                }
+                acc_tiles += nt;
+            }
+            if (!found) return t;                      // uniform for the whole workgroup
+            t.valid = 1;
+            t.m0 = start; t.n0 = tn * BN;
+            t.row_lo = cnt_lo; t.row_hi = cnt_hi;
+            t.bptr = p.b + (size_t)e * (size_t)p.k * (size_t)p.n;
+            t.bsptr = p.bs + (size_t)e * (size_t)(p.k / KBLK) * (size_t)p.nb;
+            t.kb_begin = 0; t.kb_end = p.k / KBLK;
+        } else {
+            const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
+            const int per_split = tiles_m * tiles_n, total = per_split * p.split_k;
+            // the gridDim.x tiles in flight together: every XCD takes a contiguous run of them
+            const int first = it * G;
+            const int here = total - first < G ? total - first : G;
+            if (here <= 0) return t;
+            const int v = first + xcd_virtual_id(blockIdx.x, G);
+            if (v >= total) return t;
+            (void)here;
+            t.valid = 1;
+            t.split_z = v / per_split;
+            int tm, tn;
+            band_tile(v - t.split_z * per_split, tiles_m, tiles_n, p.band_h, tm, tn);
+            t.m0 = tm * BM; t.n0 = tn * BN;
+            const int kbt = p.k / KBLK;
+            t.kb_begin = t.split_z * p.kb_per_split;
+            t.kb_end = t.kb_begin + p.kb_per_split;
+            t.kb_end = t.kb_end < kbt ? t.kb_end : kbt;
+        }
+        return t;
+    };
 
     // ---- buffer resources: out-of-range lanes read zeros instead of faulting -------------------
     const uint32_t a_bytes = (uint32_t)p.k * (uint32_t)p.lda;
     const uint32_t b_bytes = (uint32_t)p.k * (uint32_t)p.n;
     __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, a_bytes, 0x00020000);
-    __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)bptr, 0, b_bytes, 0x00020000);
+    __amdgpu_buffer_rsrc_t as_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.as, 0, (uint32_t)(p.k / KBLK) * (uint32_t)p.lda * 4u, 0x00020000);
 
-    // ---- global -> LDS copy plan --------------------------------------------------------------
+    // ---- global -> LDS copy plan of a tile -------------------------------------------------------
     // Wave w, copy q fills the 1 KiB of LDS that starts at chunk slot (q*NWAVES + w)*64; lane l fills
     // slot P = that + l, which holds k row P/CPR, stored chunk P%CPR = logical chunk (P%CPR) ^ swz(k row).
     // The XOR mask of a lane does not depend on q, so a lane's global offset is one constant (k row of
     // copy 0, chunk column) plus a wave-uniform term (k block and q), which travels in an SGPR.
     // Chunk columns beyond the matrix are clamped to its last 16 rows: such rows are never stored,
     // and every address the copies form stays inside the operand.
-    constexpr int ROWS_PER_COPY_A = C::NWAVES * 64 / C::CPR_A, ROWS_PER_COPY_B = C::NWAVES * 64 / C::CPR_B;
-    uint32_t a_voff, b_voff;
-    {
-        int P = wave * 64 + lane;
-        int krow = P / C::CPR_A, c = (P % C::CPR_A) ^ swz_of_krow<C::CPR_A>(krow);
-        int col = m0 + 16 * c;
-        col = col < p.lda - 16 ? col : p.lda - 16;
-        a_voff = (uint32_t)krow * (uint32_t)p.lda + (uint32_t)col;
-        krow = P / C::CPR_B; c = (P % C::CPR_B) ^ swz_of_krow<C::CPR_B>(krow);
-        col = n0 + 16 * c;
-        col = col < p.n - 16 ? col : p.n - 16;
-        b_voff = (uint32_t)krow * (uint32_t)p.n + (uint32_t)col;
-    }
     // a_scale row of a k block: BM floats, copied 64 floats (one dword per lane) per wave into the tail
     // of the stage.  Every wave issues the copy (wave w the same 64 floats as wave w % (BM/64), to the
     // same place): a branch here would split the K loop's straight-line block and the compiler would
     // sink the folds of the first MFMAs below it, away from the MFMAs they are meant to overlap.
+    constexpr int ROWS_PER_COPY_A = C::NWAVES * 64 / C::CPR_A, ROWS_PER_COPY_B = C::NWAVES * 64 / C::CPR_B;
     constexpr int AS_COPIES = BM / 64;
     const int as_wave = wave % AS_COPIES;
-    uint32_t as_voff;
-    {
-        int r = m0 + as_wave * 64 + lane;
+    struct CopyPlan {
+        uint32_t a_voff, b_voff, as_voff;
+        int kb_begin;
+        __amdgpu_buffer_rsrc_t b_rsrc;
+    };
+    auto copy_plan = [&](const Tile& t) -> CopyPlan {
+        CopyPlan c;
+        int P = wave * 64 + lane;
+        int krow = P / C::CPR_A, ch = (P % C::CPR_A) ^ swz_of_krow<C::CPR_A>(krow);
+        int col = t.m0 + 16 * ch;
+        col = col < p.lda - 16 ? col : p.lda - 16;
+        c.a_voff = (uint32_t)krow * (uint32_t)p.lda + (uint32_t)col;
+        krow = P / C::CPR_B; ch = (P % C::CPR_B) ^ swz_of_krow<C::CPR_B>(krow);
+        col = t.n0 + 16 * ch;
+        col = col < p.n - 16 ? col : p.n - 16;
+        c.b_voff = (uint32_t)krow * (uint32_t)p.n + (uint32_t)col;
+        int r = t.m0 + as_wave * 64 + lane;
         r = r < p.lda - 1 ? r : p.lda - 1;
-        as_voff = (uint32_t)r * 4u;
-    }
-    __amdgpu_buffer_rsrc_t as_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.as, 0, (uint32_t)(p.k / KBLK) * (uint32_t)p.lda * 4u, 0x00020000);
+        c.as_voff = (uint32_t)r * 4u;
+        c.kb_begin = t.kb_begin;
+        c.b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.bptr, 0, b_bytes, 0x00020000);
+        return c;
+    };
     const uint32_t a_kstep = (uint32_t)KBLK * (uint32_t)p.lda, b_kstep = (uint32_t)KBLK * (uint32_t)p.n;
 
     // The copies are issued from inline assembly so that the compiler's hazard tracking does not see
@@ -232,23 +268,23 @@ void gemm_tr_kernel(const GemmArgs p) {
     // enforced by hand: s_waitcnt vmcnt(0) + workgroup barrier before the first read of a stage.
     const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
     constexpr int NLOADS = C::A_LOADS + C::B_LOADS + 1;     // + the a_scale row
-    // copy q (compile-time) of k block `blk` (relative to kb_begin) into `stage`
-    auto issue_one = [&](int stage, int blk, auto q_tag) {
+    // copy q (compile-time) of k block `blk` (relative to the tile's first) into `stage`
+    auto issue_one = [&](const CopyPlan& cp, int stage, int blk, auto q_tag) {
         constexpr int q = decltype(q_tag)::value;
         const uint32_t sa = lds_base + stage * C::STAGE_BYTES + wave * 1024;
-        const uint32_t kb = (uint32_t)(kb_begin + blk);
+        const uint32_t kb = (uint32_t)(cp.kb_begin + blk);
         if constexpr (q < C::A_LOADS) {
-            copy16_global_to_lds(a_rsrc, sa + q * C::NWAVES * 1024, a_voff, kb * a_kstep + (uint32_t)(q * ROWS_PER_COPY_A) * (uint32_t)p.lda);
+            copy16_global_to_lds(a_rsrc, sa + q * C::NWAVES * 1024, cp.a_voff, kb * a_kstep + (uint32_t)(q * ROWS_PER_COPY_A) * (uint32_t)p.lda);
         } else if constexpr (q < C::A_LOADS + C::B_LOADS) {
             constexpr int qb = q - C::A_LOADS;
-            copy16_global_to_lds(b_rsrc, sa + C::A_BYTES + qb * C::NWAVES * 1024, b_voff, kb * b_kstep + (uint32_t)(qb * ROWS_PER_COPY_B) * (uint32_t)p.n);
+            copy16_global_to_lds(cp.b_rsrc, sa + C::A_BYTES + qb * C::NWAVES * 1024, cp.b_voff, kb * b_kstep + (uint32_t)(qb * ROWS_PER_COPY_B) * (uint32_t)p.n);
         } else {
-            copy4_global_to_lds(as_rsrc, lds_base + stage * C::STAGE_BYTES + C::A_BYTES + C::B_BYTES + as_wave * 256, as_voff, kb * (uint32_t)p.lda * 4u);
+            copy4_global_to_lds(as_rsrc, lds_base + stage * C::STAGE_BYTES + C::A_BYTES + C::B_BYTES + as_wave * 256, cp.as_voff, kb * (uint32_t)p.lda * 4u);
         }
     };
-    auto issue_all = [&](int stage, int blk) {
+    auto issue_all = [&](const CopyPlan& cp, int stage, int blk) {
         [&]<int... Q>(std::integer_sequence<int, Q...>) {
-            (issue_one(stage, blk, std::integral_constant<int, Q>{}), ...);
+            (issue_one(cp, stage, blk, std::integral_constant<int, Q>{}), ...);
         }(std::make_integer_sequence<int, NLOADS>{});
     };
 
@@ -278,11 +314,20 @@ void gemm_tr_kernel(const GemmArgs p) {
         }
     };
 
+    const int as_lane_off = C::A_BYTES + C::B_BYTES + (wave_m * WM + i16) * 4;
+
+    Tile cur = pick_tile(0);
+    if (!cur.valid) return;
+    CopyPlan cp = copy_plan(cur);
+    bool prefetched = false;                // block 0 of `cur` is already on its way into stage 0
+    for (int it = 0;; it++) {
+    const int m0 = cur.m0, n0 = cur.n0, kb_begin = cur.kb_begin, kb_end = cur.kb_end, split_z = cur.split_z;
+    const int row_lo = cur.row_lo, row_hi = cur.row_hi;
+    const float* bsptr = cur.bsptr;
     // ---- scales -------------------------------------------------------------------------------
     // a_scale: lane's output row of m-tile t is tile row wave_m*WM + 16t + i16, read from the stage's
     // copy of the a_scale row.  b_scale: one value per wave and k block (a wave's n range lies inside
     // one 128-block), loaded straight from memory two k blocks ahead.
-    const int as_lane_off = C::A_BYTES + C::B_BYTES + (wave_m * WM + i16) * 4;
     int nblk = (n0 + wave_n * WN) / 128;
     nblk = __builtin_amdgcn_readfirstlane(nblk < p.nb - 1 ? nblk : p.nb - 1);
 
@@ -304,16 +349,18 @@ void gemm_tr_kernel(const GemmArgs p) {
         constexpr int DMA_EVERY = (STEPS - C::MT) / NL_EARLY >= 2 ? 2 : 1, DMA_FIRST = DMA_EVERY - 1;
         static_assert(NL_EARLY * DMA_EVERY <= STEPS - C::MT, "not enough steps to issue the copies before the barrier");
 
-        // ---- prologue: block 0 -> stage 0, wait; first copies of block 1 -> stage 1 ----
+        // ---- prologue: block 0 -> stage 0 (unless the previous tile already sent it), wait; first
+        //      copies of block 1 -> stage 1.  The barrier also ends the previous tile's use of stage 1
+        //      as the staging area of its output ----
         const float* bs_ptr = bsptr + (size_t)kb_begin * p.nb + nblk;   // b_scale of the current k block
         float bs_cur = bs_ptr[0];
         float bs_nxt = nkb > 1 ? bs_ptr[p.nb] : 0.f;
-        issue_all(0, 0);
+        if (!prefetched) issue_all(cp, 0, 0);
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
         __syncthreads();
         if (nkb > 1) {
             [&]<int... Q>(std::integer_sequence<int, Q...>) {
-                (issue_one(1, 1, std::integral_constant<int, Q>{}), ...);
+                (issue_one(cp, 1, 1, std::integral_constant<int, Q>{}), ...);
             }(std::make_integer_sequence<int, NL_LATE>{});
         }
 
@@ -341,7 +388,7 @@ void gemm_tr_kernel(const GemmArgs p) {
                 if constexpr (s < STEPS) {
                     constexpr int u = s / C::MT, t = s % C::MT;
                     if constexpr (HAS_NEXT && s % DMA_EVERY == DMA_FIRST && s / DMA_EVERY < NL_EARLY)
-                        issue_one(cur_stage ^ 1, j + 1, std::integral_constant<int, NL_LATE + s / DMA_EVERY>{});
+                        issue_one(cp, cur_stage ^ 1, j + 1, std::integral_constant<int, NL_LATE + s / DMA_EVERY>{});
                     if constexpr (t == 0 && u + 1 < C::NT) read_b(breg[(u + 1) & 1], u + 1, sbase);
                     if constexpr (t == 0 && u == C::NT - 1) {
                         // All reads of this stage are issued.  Wait for them and for this wave's part
@@ -358,7 +405,7 @@ void gemm_tr_kernel(const GemmArgs p) {
                         if constexpr (t == 0) read_b(breg[0], 0, snext);
                     }
                     if constexpr (u == C::NT - 1 && HAS_NEXT2 && t < NL_LATE)
-                        issue_one(cur_stage, j + 2, std::integral_constant<int, t>{});
+                        issue_one(cp, cur_stage, j + 2, std::integral_constant<int, t>{});
                 }
                 if constexpr (s >= LAG) {
                     constexpr int sp = s - LAG, u = sp / C::MT, t = sp % C::MT;
@@ -378,6 +425,20 @@ void gemm_tr_kernel(const GemmArgs p) {
         k_block(j, std::false_type{}, std::false_type{});
     }
 
+    else if (it > 0) {
+        __syncthreads();                    // nothing to multiply: still let the previous tile's staging reads finish
+    }
+
+    // ---- the next tile's first K block starts now: after the last barrier above no wave reads a
+    //      stage any more, and the output below is staged in stage 1 only ----
+    Tile nxt = pick_tile(it + 1);
+    CopyPlan ncp = cp;
+    prefetched = false;
+    if (nxt.valid) {
+        ncp = copy_plan(nxt);
+        if (nxt.kb_end > nxt.kb_begin) { issue_all(ncp, 0, 0); prefetched = true; }
+    }
+
     // ---- epilogue -----------------------------------------------------------------------------
     if (MODE == 1) {
         // split-K: fp32 partial tile, 16 bytes per lane
@@ -394,46 +455,58 @@ void gemm_tr_kernel(const GemmArgs p) {
         }
     } else {
         // bf16 through LDS so that the global stores are 16 bytes per lane and every store
-        // instruction writes whole rows of the wave tile (WN*2 contiguous bytes each).  The stages are
-        // free: after the barrier of the last K block no wave reads them and no copy is in flight.
-        // Each wave uses its own WM x WN bf16 region; 16-byte chunks are XOR-swizzled by row so that
-        // neither the 8-byte writes (16 rows per instruction) nor the 16-byte reads conflict.
+        // instruction writes whole rows of the wave tile (WNO*2 contiguous bytes each).  Stage 1 is
+        // free (after the barrier of the last K block no wave reads it and no copy into it is in
+        // flight); stage 0 already receives the next tile.  Each wave stages its tile in two halves of
+        // WM/2 rows in its own region; 16-byte chunks are XOR-swizzled by row so that neither the
+        // writes (16 rows per instruction) nor the 16-byte reads conflict.
         constexpr int WNO = EPI == 1 ? WN / 2 : WN;                   // output columns of the wave tile
         constexpr int ROW_CHUNKS = WNO * 2 / 16;                      // 16-byte chunks per tile row
         constexpr int ROWS_PER_SWEEP = 16 / ROW_CHUNKS > 0 ? 16 / ROW_CHUNKS : 1;
-        unsigned char* region = lds + wave * (WM * WNO * 2);
-#pragma unroll
-        for (int t = 0; t < C::MT; t++) {
-            const int r = 16 * t + i16;
-            const int sw = (r / ROWS_PER_SWEEP) % ROW_CHUNKS;
-#pragma unroll
-            for (int u = 0; u < C::NT; u++) {
-                if (EPI == 1) {
-                    // the lane's four columns are two (gate, up) pairs -> two outputs, 4 bytes
-                    const uint32_t o = pack_bf16x2(silu_mul(acc[t][u][0], acc[t][u][1]), silu_mul(acc[t][u][2], acc[t][u][3]));
-                    *(uint32_t*)(region + r * (WNO * 2) + ((u ^ sw) << 4) + g * 4) = o;
-                } else {
-                    v2i o;
-                    o[0] = (int)pack_bf16x2(acc[t][u][0], acc[t][u][1]);
-                    o[1] = (int)pack_bf16x2(acc[t][u][2], acc[t][u][3]);
-                    const int chunk = 2 * u + (g >> 1);
-                    *(v2i*)(region + r * (WNO * 2) + ((chunk ^ sw) << 4) + (g & 1) * 8) = o;
-                }
-            }
-        }
-        constexpr int PASSES = WM * ROW_CHUNKS / 64;
+        constexpr int HALF_ROWS = WM / 2, HALF_MT = C::MT / 2;
+        static_assert(C::MT % 2 == 0 && C::NWAVES * HALF_ROWS * WNO * 2 <= C::STAGE_BYTES, "output staging must fit one stage");
+        unsigned char* region = lds + C::STAGE_BYTES + wave * (HALF_ROWS * WNO * 2);
         const int ldc = EPI == 1 ? p.n / 2 : p.n;
 #pragma unroll
-        for (int q = 0; q < PASSES; q++) {
-            const int idx = q * 64 + lane;
-            const int r = idx / ROW_CHUNKS, chunk = idx % ROW_CHUNKS;
-            const int sw = (r / ROWS_PER_SWEEP) % ROW_CHUNKS;
-            const v4i val = *(const v4i*)(region + r * (WNO * 2) + ((chunk ^ sw) << 4));
-            const int row = m0 + wave_m * WM + r, col = (EPI == 1 ? (n0 + wave_n * WN) / 2 : n0 + wave_n * WN) + chunk * 8;
-            if (row >= row_lo && row < row_hi && col < ldc)
-                *(v4i*)(p.c + (size_t)row * ldc + col) = val;
+        for (int half = 0; half < 2; half++) {
+#pragma unroll
+            for (int th = 0; th < HALF_MT; th++) {
+                const int t = half * HALF_MT + th;
+                const int r = 16 * th + i16;
+                const int sw = (r / ROWS_PER_SWEEP) % ROW_CHUNKS;
+#pragma unroll
+                for (int u = 0; u < C::NT; u++) {
+                    if (EPI == 1) {
+                        // the lane's four columns are two (gate, up) pairs -> two outputs, 4 bytes
+                        const uint32_t o = pack_bf16x2(silu_mul(acc[t][u][0], acc[t][u][1]), silu_mul(acc[t][u][2], acc[t][u][3]));
+                        *(uint32_t*)(region + r * (WNO * 2) + ((u ^ sw) << 4) + g * 4) = o;
+                    } else {
+                        v2i o;
+                        o[0] = (int)pack_bf16x2(acc[t][u][0], acc[t][u][1]);
+                        o[1] = (int)pack_bf16x2(acc[t][u][2], acc[t][u][3]);
+                        const int chunk = 2 * u + (g >> 1);
+                        *(v2i*)(region + r * (WNO * 2) + ((chunk ^ sw) << 4) + (g & 1) * 8) = o;
+                    }
+                }
+            }
+            constexpr int PASSES = HALF_ROWS * ROW_CHUNKS / 64;
+            static_assert(HALF_ROWS * ROW_CHUNKS % 64 == 0, "a half tile is a whole number of 16-byte sweeps");
+#pragma unroll
+            for (int q = 0; q < PASSES; q++) {
+                const int idx = q * 64 + lane;
+                const int r = idx / ROW_CHUNKS, chunk = idx % ROW_CHUNKS;
+                const int sw = (r / ROWS_PER_SWEEP) % ROW_CHUNKS;
+                const v4i val = *(const v4i*)(region + r * (WNO * 2) + ((chunk ^ sw) << 4));
+                const int row = m0 + wave_m * WM + half * HALF_ROWS + r;
+                const int col = (EPI == 1 ? (n0 + wave_n * WN) / 2 : n0 + wave_n * WN) + chunk * 8;
+                if (row >= row_lo && row < row_hi && col < ldc)
+                    *(v4i*)(p.c + (size_t)row * ldc + col) = val;
+            }
         }
     }
+    if (!nxt.valid) break;
+    cur = nxt; cp = ncp;
+    }   // tiles
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -709,32 +782,47 @@ static hipError_t launch_tr(const GemmArgs& a, dim3 grid, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// CUs of the current device (asked once per process and device change is not expected mid-run)
+static int device_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+        else cus = 256;
+    }
+    return cus;
+}
+
 template <int BM, int BN, int WM, int WN, bool WITH_EPI = false>
 static hipError_t launch_shape(const GemmArgs& a, int mode, hipStream_t stream) {
+    using C = TileCfg<BM, BN, WM, WN, 0>;
+    // persistent workgroups: as many as fit the chip at once (LDS and thread limits), each walks
+    // tiles  blockIdx.x, blockIdx.x + grid, ...
+    const int by_lds = 163840 / C::LDS_BYTES, by_threads = 2048 / C::NTHREADS;
+    const long resident = (long)device_cus() * (by_lds < by_threads ? by_lds : by_threads);
+    const int tiles_n = (a.n + BN - 1) / BN;
+    long total;
+    if (mode == 2) {
+        // upper bound on m-tile slots: every expert can waste up to 15 rows (aligned-down start)
+        // plus one partial tile; workgroups beyond the real count find no tile and leave
+        total = (((long)a.m + BM - 1) / BM + 2L * a.num_experts) * tiles_n;
+    } else {
+        total = (long)((a.m + BM - 1) / BM) * tiles_n * a.split_k;
+    }
+    const dim3 grid((unsigned)(total < resident ? total : resident));
     if (a.epi != 0) {
         // the fused silu-mul epilogue exists for the 256x256 tile, dense or grouped, without K split
         if constexpr (WITH_EPI) {
-            int tiles_n = (a.n + BN - 1) / BN;
             if (a.epi != 1 || mode == 1) return hipErrorInvalidValue;
-            if (mode == 2) {
-                long slots = ((long)a.m + BM - 1) / BM + 2L * a.num_experts;
-                return launch_tr<BM, BN, WM, WN, 2, 1>(a, dim3(tiles_n, (unsigned)slots), stream);
-            }
-            return launch_tr<BM, BN, WM, WN, 0, 1>(a, dim3(((a.m + BM - 1) / BM) * tiles_n), stream);
+            if (mode == 2) return launch_tr<BM, BN, WM, WN, 2, 1>(a, grid, stream);
+            return launch_tr<BM, BN, WM, WN, 0, 1>(a, grid, stream);
         } else {
             return hipErrorInvalidValue;
         }
     }
-    if (mode == 2) {
-        int tiles_n = (a.n + BN - 1) / BN;
-        // upper bound on m-tile slots: every expert can waste up to 15 rows (aligned-down start)
-        // plus one partial tile
-        long slots = ((long)a.m + BM - 1) / BM + 2L * a.num_experts;
-        return launch_tr<BM, BN, WM, WN, 2>(a, dim3(tiles_n, (unsigned)slots), stream);
-    }
-    int tiles = ((a.m + BM - 1) / BM) * ((a.n + BN - 1) / BN) * a.split_k;
-    if (mode == 1) return launch_tr<BM, BN, WM, WN, 1>(a, dim3(tiles), stream);
-    return launch_tr<BM, BN, WM, WN, 0>(a, dim3(tiles), stream);
+    if (mode == 2) return launch_tr<BM, BN, WM, WN, 2>(a, grid, stream);
+    if (mode == 1) return launch_tr<BM, BN, WM, WN, 1>(a, grid, stream);
+    return launch_tr<BM, BN, WM, WN, 0>(a, grid, stream);
 }
 
 hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t stream) {
