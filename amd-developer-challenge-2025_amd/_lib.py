@@ -15,7 +15,7 @@ EXPORTS = (
     "fp8bs_gemm", "fp8bs_gemm_ex", "fp8bs_gemm_grouped",
     "fp8bs_quantize_a", "fp8bs_quantize_b",
     "fp8bs_moe_topk", "fp8bs_moe_route_workspace_bytes", "fp8bs_moe_route",
-    "fp8bs_gemm_silu_mul", "fp8bs_moe_combine",
+    "fp8bs_gemm_silu_mul", "fp8bs_moe_combine", "fp8bs_convert_fnuz_to_fn",
 )
 
 VARIANT_NAMES = {0: "auto", 1: "generic", 2: "t256x256", 3: "t128x128", 4: "t64x128", 5: "t256x128", 6: "skinny64x144"}
@@ -74,6 +74,8 @@ def load() -> ctypes.CDLL:
     lib.fp8bs_gemm_silu_mul.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]
     lib.fp8bs_moe_combine.restype = i32
     lib.fp8bs_moe_combine.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
+    lib.fp8bs_convert_fnuz_to_fn.restype = i32
+    lib.fp8bs_convert_fnuz_to_fn.argtypes = [vp, vp, sz, vp]
     _lib = lib
     return lib
 

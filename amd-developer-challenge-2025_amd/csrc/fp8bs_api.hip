@@ -63,36 +63,41 @@ void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     if ((m % 16) != 0 || (n % 16) != 0) { fill_plan(m, n, k, FP8BS_VARIANT_GENERIC, 1, out); return; }
     int kbt = k / KBLK;
     if (m > 128) {
-        // Compute-bound family.  Cost model in units of "one 256x256 tile over all of K on a CU of its
-        // own": rounds over the chip x workgroups sharing a CU x tile area x a measured per-area
-        // penalty (smaller tiles re-read more of A and B from LDS per multiply).
-        struct Cand { int variant; int wgs_per_cu; double area, penalty; };
-        const Cand cands[3] = {
-            {FP8BS_VARIANT_T256x256, 1, 1.0, 1.0},
-            {FP8BS_VARIANT_T256x128, 1, 0.5, 1.16},
-            {FP8BS_VARIANT_T128x128, 2, 0.25, 1.29},
+        // Compute-bound family: the tile shape and K split that finish soonest under a cost model in
+        // microseconds.  Per variant and number r of workgroups resident on a CU, measured on MI355X
+        // (K = 1024 and 8192 on shapes of exactly r workgroups per CU): the time in which all r advance
+        // one K block, and the fixed time of a round (prologue, output, drain).  Workgroups are dealt in
+        // rounds of (CUs x the most that fit a CU); a last partial round runs with fewer per CU.  A K
+        // split adds the fp32 partial planes (written and read back, mostly through the 256 MB cache) and the
+        // reduce launch.
+        struct Cand { int variant; int rmax; double t_block[3], t_fixed[3]; };
+        const Cand cands[4] = {
+            {FP8BS_VARIANT_T256x256, 1, {1.87, 0, 0}, {6.8, 0, 0}},
+            {FP8BS_VARIANT_T256x128, 1, {1.22, 0, 0}, {4.4, 0, 0}},
+            {FP8BS_VARIANT_T128x128, 2, {0.89, 1.34, 0}, {3.1, 4.8, 0}},
+            {FP8BS_VARIANT_T64x128, 3, {0.70, 1.04, 1.39}, {1.9, 2.3, 3.6}},
         };
-        int best_variant = 0; double best_cost = 0;
+        const int splits[6] = {1, 2, 3, 4, 6, 8};
+        int best_variant = 0, best_split = 1; double best_cost = 0;
         for (const Cand& c : cands) {
             VariantInfo vi{};
             variant_info(c.variant, &vi);
-            long tiles = cdiv(m, vi.bm) * cdiv(n, vi.bn);
-            double cost = (double)cdiv(tiles, (long)num_cus * c.wgs_per_cu) * c.wgs_per_cu * c.area * c.penalty;
-            if (best_variant == 0 || cost < best_cost) { best_variant = c.variant; best_cost = cost; }
+            const long tiles = cdiv(m, vi.bm) * cdiv(n, vi.bn);
+            for (int s : splits) {
+                if (s > 1 && kbt / s < 4) continue;                  // keep at least 4 K blocks per workgroup
+                const long wgs = tiles * s, per_round = (long)num_cus * c.rmax;
+                const long full = wgs / per_round, rem = wgs % per_round;
+                const double kb = (double)cdiv(kbt, s);
+                double cost = (double)full * (c.t_fixed[c.rmax - 1] + kb * c.t_block[c.rmax - 1]);
+                if (rem) {
+                    const long r = cdiv(rem, num_cus);
+                    cost += c.t_fixed[r - 1] + kb * c.t_block[r - 1];
+                }
+                if (s > 1) cost += 2.0 + 8.0 * s * (double)m * (double)n / 8.0e6;
+                if (best_variant == 0 || cost < best_cost) { best_variant = c.variant; best_split = s; best_cost = cost; }
+            }
         }
-        VariantInfo vi{};
-        variant_info(best_variant, &vi);
-        long tiles = cdiv(m, vi.bm) * cdiv(n, vi.bn);
-        // split K only when the tiles cover less than half of the chip and K is long
-        int s = 1;
-        if (tiles * 2 <= num_cus && kbt >= 8) {
-            long want = num_cus / tiles;
-            long max_split = kbt / 4;
-            s = (int)(want > max_split ? max_split : want);
-            if (s > 8) s = 8;
-            if (s < 1) s = 1;
-        }
-        fill_plan(m, n, k, best_variant, s, out);
+        fill_plan(m, n, k, best_variant, best_split, out);
         return;
     }
     {

@@ -238,7 +238,44 @@ static hipError_t launch_quant(const QuantArgs& a, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// e4m3fnuz (gfx942: bias 8, max 240, NaN = 0x80, no -0) -> e4m3fn (bias 7) with the same value.
+// Normal fnuz codes with exponent field >= 2 are the fn code with the exponent field one lower, exactly.
+// The 16 smallest magnitudes (fnuz subnormals and exponent field 1, steps of 2^-10) fall on fn's
+// subnormal grid of 2^-9: magnitude code x becomes x/2 rounded to nearest even.  16 bytes per thread.
+__device__ __forceinline__ uint32_t fnuz_to_fn_byte(uint32_t b) {
+    const uint32_t mag = b & 0x7Fu;
+    const uint32_t out = mag >= 16u ? mag - 8u : (mag + ((mag >> 1) & 1u)) >> 1;
+    return b == 0x80u ? 0x7Fu : ((b & 0x80u) | out);
+}
+__global__ __launch_bounds__(256)
+void fnuz_to_fn_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, size_t n) {
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 16;
+    if (i + 16 <= n) {
+        const v4i v = *(const v4i*)(src + i);
+        v4i o;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const uint32_t x = (uint32_t)v[w];
+            o[w] = (int)(fnuz_to_fn_byte(x & 0xFFu) | (fnuz_to_fn_byte((x >> 8) & 0xFFu) << 8) |
+                         (fnuz_to_fn_byte((x >> 16) & 0xFFu) << 16) | (fnuz_to_fn_byte(x >> 24) << 24));
+        }
+        *(v4i*)(dst + i) = o;
+    } else {
+        for (size_t j = i; j < n; j++) dst[j] = (uint8_t)fnuz_to_fn_byte(src[j]);
+    }
+}
+
 }  // namespace fp8bs
+
+extern "C" int fp8bs_convert_fnuz_to_fn(const void* src, void* dst, size_t nbytes, void* stream) {
+    if (nbytes == 0) return FP8BS_OK;
+    if (!src || !dst) return FP8BS_ERR_NULL_POINTER;
+    if ((((uintptr_t)src | (uintptr_t)dst) & 15) != 0) return FP8BS_ERR_BAD_SHAPE;
+    const size_t threads = (nbytes + 15) / 16;
+    hipLaunchKernelGGL(fp8bs::fnuz_to_fn_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint8_t*)src, (uint8_t*)dst, nbytes);
+    return hipGetLastError() == hipSuccess ? FP8BS_OK : FP8BS_ERR_LAUNCH;
+}
 
 namespace {
 int quantize_common(const void* x, int dtype, int64_t ldx, const int32_t* row_map, int src_rows, void* q, float* scale,

@@ -34,8 +34,24 @@ def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
 
 
 def _is_kmajor(t: torch.Tensor) -> bool:
-    """True if the 2-D tensor's storage is its transpose laid out contiguously (stride (1, rows))."""
-    return t.dim() == 2 and t.t().is_contiguous()
+    """True if the 2-D tensor's storage is its transpose laid out contiguously (stride (1, rows));
+    the stride of a dimension of size 1 is immaterial."""
+    if t.dim() != 2:
+        return False
+    r, c = t.shape
+    s0, s1 = t.stride()
+    return r == 0 or c == 0 or ((r == 1 or s0 == 1) and (c == 1 or s1 == r))
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_plan_cache = {}   # (m, n, k) -> workspace bytes the planner asks for
+
+
+def _stream_ptr(device: torch.device) -> int:
+    """Raw hipStream_t of torch's current stream on `device` (the stream the library launches on)."""
+    if _raw_stream is not None:
+        return _raw_stream(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
 
 
 def _check_operands(a, b, a_scale, b_scale, c, rows, n, k):
@@ -88,17 +104,24 @@ def custom_kernel(data, variant: int = 0, split_k: int = 0):
         raise ValueError("b and b_scale must be K-major (stride (1, n) / (1, ceil(n/128)))")
     lib = _lib.load()
     if variant == 0 and split_k == 0:
-        need = workspace_bytes(m, n, k) if (m > 0 and n > 0 and k > 0) else 0
+        need = _plan_cache.get((m, n, k))
+        if need is None:
+            need = workspace_bytes(m, n, k) if (m > 0 and n > 0 and k > 0) else 0
+            _plan_cache[(m, n, k)] = need
     else:
         need = max(split_k, 1) * m * n * 4 if split_k > 1 else 0
     ws_ptr, ws_len = None, 0
     if need:
         ws = _workspace(a.device, need)
         ws_ptr, ws_len = ws.data_ptr(), ws.numel()
-    with torch.cuda.device(a.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    # kernels are launched on the device the pointers live on: the library uses the current device
+    if a.device.index != torch.cuda.current_device():
+        with torch.cuda.device(a.device):
+            st = lib.fp8bs_gemm_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
+                                   c.data_ptr(), ws_ptr, ws_len, m, n, k, variant, split_k, _stream_ptr(a.device))
+    else:
         st = lib.fp8bs_gemm_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
-                               c.data_ptr(), ws_ptr, ws_len, m, n, k, variant, split_k, stream)
+                               c.data_ptr(), ws_ptr, ws_len, m, n, k, variant, split_k, _stream_ptr(a.device))
     _lib.check(st)
     return c
 

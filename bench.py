@@ -260,6 +260,14 @@ def main():
                                                  "bound": "hbm", "frac": round(by / us * 1e-3 / PEAK_HBM_GBS, 4),
                                                  "note": "y (470 MB) was just written and may partly sit in the 256 MB cache"}
         dd = a2 = b2 = y = h = None
+        # the 18 shapes of the upstream benchmark the reference was ranked on (README.md:65-82); the
+        # leaderboard's score is an aggregate of the per-shape times (top three on MI300X: 103-116 us)
+        torch.cuda.empty_cache()
+        harness = importlib.import_module("amd-developer-challenge-2025_amd.harness")
+        rows_, geo = harness.benchmark(steps=max(args.steps // 2, 5), warmup=3, device=dev)
+        per_config["leaderboard_18_shapes"] = {
+            "geomean_us": round(geo, 2), "mean_us": round(sum(r["us"] for r in rows_) / len(rows_), 2),
+            "shapes": ["%dx%dx%d: %.1f us, %.0f TF" % (r["m"], r["n"], r["k"], r["us"], r["tflops"]) for r in rows_]}
     result["per_config"] = per_config
 
     # ---- CPU baseline: the oracle on the same configuration-2 inputs, host cores ----

@@ -127,6 +127,13 @@ int fp8bs_quantize_a(const void* x, int x_dtype, int64_t ldx, const int32_t* row
 int fp8bs_quantize_b(const void* w, int w_dtype, int64_t ldw, void* b, float* b_scale, int n, int k,
                      void* stream);
 
+/* e4m3fnuz bytes (the gfx942 type of the reference, 1-amd-fp8-mm/amd-fp8-mm-submission.py:20-21: bias 8,
+ * max 240, NaN 0x80) -> e4m3fn bytes of the same value, so that operands quantised for the reference's
+ * hardware can be fed to this library unchanged in scale.  Exact except for the 16 smallest magnitudes
+ * (below 2^-6), which land on e4m3fn's coarser subnormal grid with round-to-nearest-even.  src and dst
+ * must be 16-byte aligned and may be the same buffer. */
+int fp8bs_convert_fnuz_to_fn(const void* src, void* dst, size_t nbytes, void* stream);
+
 /* ---- MoE routing (the caller of the grouped GEMM) ------------------------------------------------
  * Top-k selection with the reference's rule (2-amd-moe/amd-moe-submission.py:32-56, 58-105): per token,
  * k times the strictly greatest score not yet taken, lowest index first among equals, best first; NaN

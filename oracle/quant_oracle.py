@@ -26,6 +26,9 @@ How each function is pinned (tests/test_quant_oracle.py):
                     invariants: |decoded q| <= 448, the largest |x| of every non-zero block maps to
                     code 448, relative error of normal values <= 2^-4, re-quantising the dequantised
                     values returns the same codes
+  * fnuz_to_fn_ref  (e4m3fnuz, the reference's gfx942 type, 1-amd-fp8-mm/amd-fp8-mm-submission.py:20-21:
+                    bias 8, NaN 0x80, no -0)  torch's own float8_e4m3fnuz -> float32 -> float8_e4m3fn
+                    casts on all 256 codes
 """
 import numpy as np
 
@@ -101,3 +104,18 @@ def quantize_b_ref(w: np.ndarray):
     q = np.clip(wb / scale[:, None, :, None], -FP8_MAX, FP8_MAX).astype(np.float32)
     codes = encode_e4m3fn(q.reshape(nb * BLOCK, k)[:n])
     return np.ascontiguousarray(codes.T), np.ascontiguousarray(scale.T)
+
+
+def decode_e4m3fnuz(codes: np.ndarray) -> np.ndarray:
+    """uint8 e4m3fnuz codes -> float32: (-1)^s 2^(e-8) (1 + m/8), subnormals m 2^-10, 0x80 = NaN, no -0."""
+    c = np.asarray(codes, dtype=np.uint8).astype(np.int32)
+    e, m = (c >> 3) & 15, c & 7
+    mag = np.where(e == 0, m * 2.0 ** -10, (1.0 + m / 8.0) * np.exp2(e.astype(np.float64) - 8))
+    v = np.where(c & 0x80, -mag, mag)
+    return np.where(c == 0x80, np.nan, v).astype(np.float32)
+
+
+def fnuz_to_fn_ref(codes: np.ndarray) -> np.ndarray:
+    """e4m3fnuz codes -> e4m3fn codes of the same value (round to nearest even where fn is coarser)."""
+    out = encode_e4m3fn(decode_e4m3fnuz(codes))
+    return np.where(np.asarray(codes, dtype=np.uint8) == 0x80, np.uint8(0x7F), out).astype(np.uint8)

@@ -34,8 +34,12 @@ def test_plan_shape_families(pkg):
     assert p.workspace_bytes == p.split_k * 64 * 18432 * 4 == pkg.workspace_bytes(64, 18432, 7168)
     p = pkg.plan(130, 192, 256)                         # not a multiple of 16 -> generic kernel
     assert p.variant == 1 and p.split_k == 1
-    p = pkg.plan(256, 512, 1024)
-    assert p.variant in (3, 5) and p.split_k >= 1 and p.split_k <= 8
+    p = pkg.plan(256, 512, 1024)                        # small: one of the sub-256 tiles, never the scalar kernel
+    assert p.variant in (3, 4, 5) and p.split_k >= 1 and p.split_k <= 8
+    p = pkg.plan(1024, 512, 7168)                       # few tiles, long K: the planner splits K
+    assert p.variant in (3, 4, 5) and p.split_k > 1
+    p = pkg.plan(6144, 4608, 7168)                      # large: the 256x256 tile, no split
+    assert p.variant == 2 and p.split_k == 1
 
 
 def test_plan_rejects_bad_shapes(pkg):

@@ -113,3 +113,18 @@ def test_row_map_gathers_rows(qo):
             assert np.array_equal(q[:, i], qf[:, r]) and s[0, i] == sf[0, r]
         else:
             assert not q[:, i].any() and s[0, i] == np.float32(1e-12)
+
+
+def test_fnuz_to_fn_against_torch_casts(qo):
+    codes = np.arange(256, dtype=np.uint8)
+    vals = torch.from_numpy(codes.copy()).view(torch.float8_e4m3fnuz).float()
+    assert np.array_equal(np.nan_to_num(qo.decode_e4m3fnuz(codes), nan=-777.0), np.nan_to_num(vals.numpy(), nan=-777.0))
+    want = vals.to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = qo.fnuz_to_fn_ref(codes)
+    finite = codes != 0x80
+    assert np.array_equal(got[finite], want[finite])
+    assert got[0x80] == 0x7F                                   # the fnuz NaN becomes an fn NaN
+    # exact wherever the magnitude code is >= 16
+    exact = finite & ((codes & 0x7F) >= 16)
+    tab = np.array([(((c & 0x7F) - 8) & 0x7F) | (c & 0x80) for c in range(256)], dtype=np.uint8)
+    assert np.array_equal(got[exact], tab[exact])
