@@ -26,6 +26,8 @@ bool variant_info(int variant, VariantInfo* out) {
         case FP8BS_VARIANT_T64x128:  *out = {64, 128, 256}; return true;
         case FP8BS_VARIANT_T256x128: *out = {256, 128, 512}; return true;
         case FP8BS_VARIANT_SKINNY64x144: *out = {64, 144, 256}; return true;
+        case FP8BS_VARIANT_SKINNY64x256: *out = {64, 256, 256}; return true;
+        case FP8BS_VARIANT_SKINNY64x288: *out = {64, 288, 256}; return true;
         default: return false;
     }
 }

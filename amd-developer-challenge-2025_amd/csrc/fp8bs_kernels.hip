@@ -528,15 +528,25 @@ void gemm_tr_kernel(const GemmArgs p) {
 // columns span) ride the same ring.
 //   MODE 0: bf16 output      MODE 1: fp32 split-K partial planes
 // ---------------------------------------------------------------------------------------------------
+// Tile widths: 144 (9 chunks: odd, no swizzle needed), 288 (18 chunks: the 8 k rows one 16-lane group
+// reads are still 8 different bank groups), 256 (16 chunks: XOR swizzle as in the main kernel; rows are
+// whole 128-byte lines, the cheapest for the texture path).  The copies of a block are padded with
+// repeats of the last one to the same number per wave, which makes "block j has landed" a fixed
+// s_waitcnt vmcnt threshold.
+template <int BN_, int NSTAGE_>
 struct SkinnyCfg {
-    static constexpr int BM = 64, BN = 144, CPR_A = 4, CPR_B = 9, NWAVES = 4, NTHREADS = 256;
+    static constexpr int BM = 64, BN = BN_, CPR_A = 4, CPR_B = BN / 16, NWAVES = 4, NTHREADS = 256;
+    static constexpr bool SWZ_B = (CPR_B % 2 == 0) && (CPR_B != 18);
     static constexpr int A_BYTES = KBLK * BM, B_BYTES = KBLK * BN, SC_BYTES = 1024;
-    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + SC_BYTES;      // 27 KiB
-    static constexpr int NSTAGE = 4;
-    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;               // 108 KiB
-    static constexpr int COPIES = 7;                                      // per wave per K block
-    static constexpr int MT = BM / 16, NT_MAX = 3;                        // n tiles per wave: ceil(9 / 4)
-    static_assert(A_BYTES / 1024 + B_BYTES / 1024 + 2 == COPIES * NWAVES, "copy plan must cover a block exactly");
+    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + SC_BYTES;
+    static constexpr int NSTAGE = NSTAGE_;
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
+    static constexpr int A_COPIES = A_BYTES / 1024, B_COPIES = B_BYTES / 1024;
+    static constexpr int COPIES = (A_COPIES + B_COPIES + 2 + NWAVES - 1) / NWAVES;     // per wave per K block
+    static constexpr int MT = BM / 16, NT_MAX = (CPR_B + NWAVES - 1) / NWAVES;        // n tiles per wave
+    static_assert(!SWZ_B || CPR_B == 16, "the XOR swizzle is written for 256-byte rows");
+    static_assert((NSTAGE - 2) * COPIES <= 63, "vmcnt has 6 bits");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS");
 };
 
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
@@ -544,18 +554,18 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <int MODE>
+template <int BN_, int NSTAGE_, int MODE>
 __global__ __launch_bounds__(256)
 void gemm_skinny_kernel(const GemmArgs p) {
-    using C = SkinnyCfg;
+    using C = SkinnyCfg<BN_, NSTAGE_>;
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 4, i16 = lane & 15;
 
     const int tiles_n = (p.n + C::BN - 1) / C::BN;
-    // neighbouring n tiles share 128-byte lines of every k row of B (144 is not a multiple of 128):
-    // give each XCD a contiguous run of tiles so that the shared lines are fetched into one L2 only
+    // neighbouring n tiles can share 128-byte lines of every k row of B: give each XCD a contiguous
+    // run of tiles so that the shared lines are fetched into one L2 only
     const int bid = xcd_virtual_id(blockIdx.x, gridDim.x);
     const int tn = bid % tiles_n, split_z = (bid / tiles_n) % p.split_k, tm = bid / (tiles_n * p.split_k);
     const int m0 = tm * C::BM, n0 = tn * C::BN;
@@ -571,46 +581,57 @@ void gemm_skinny_kernel(const GemmArgs p) {
     __amdgpu_buffer_rsrc_t as_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.as, 0, (uint32_t)kbt * (uint32_t)p.lda * 4u, 0x00020000);
     __amdgpu_buffer_rsrc_t bs_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.bs, 0, (uint32_t)kbt * (uint32_t)p.nb * 4u, 0x00020000);
 
-    // ---- copy plan.  The 28 one-KiB copies of a block are numbered I = 4q + wave, q = 0..6:
-    //      I 0..7 the A tile, 8..25 the B tile (copy Ib = I - 8 fills B chunks 64*Ib ..), 26 the a_scale
-    //      row, 27 the b_scale values.  Lane offsets are fixed for the whole kernel; the K block enters
-    //      through the wave-uniform offset.  Columns beyond the matrix are clamped (never stored).
-    uint32_t a_voff, b_voff[5], sc_voff = 0;
-    {
-        int krow = lane / 4;                                       // + 16*I
-        int c = (lane % 4) ^ swz_of_krow<C::CPR_A>(krow);          // the XOR mask does not depend on I
-        int col = m0 + 16 * c;
-        col = col < p.lda - 16 ? col : p.lda - 16;
-        a_voff = (uint32_t)krow * (uint32_t)p.lda + (uint32_t)col;
+    // ---- copy plan.  The one-KiB copies of a block are numbered I = 4q + wave, q = 0..COPIES-1:
+    //      I < A_COPIES the A tile, then B_COPIES of the B tile (copy Ib fills B chunks 64*Ib ..), then the
+    //      a_scale row, then the b_scale values (repeated as padding).  Lane offsets are fixed for the
+    //      whole kernel; the K block enters through the wave-uniform offset.  Columns beyond the matrix
+    //      are clamped (never stored).
+    uint32_t voff[C::COPIES];
 #pragma unroll
-        for (int i = 0; i < 5; i++) {
-            int P = 64 * (4 * i + wave) + lane;
+    for (int q = 0; q < C::COPIES; q++) {
+        const int I = 4 * q + wave;
+        uint32_t v;
+        if (I < C::A_COPIES) {
+            int krow = 16 * I + lane / 4;
+            int c = (lane % 4) ^ swz_of_krow<C::CPR_A>(krow);
+            int col = m0 + 16 * c;
+            col = col < p.lda - 16 ? col : p.lda - 16;
+            v = (uint32_t)krow * (uint32_t)p.lda + (uint32_t)col;
+        } else if (I < C::A_COPIES + C::B_COPIES) {
+            int P = 64 * (I - C::A_COPIES) + lane;
             int kr = P / C::CPR_B, cc = P % C::CPR_B;
+            if (C::SWZ_B) cc ^= swz_of_krow<C::CPR_B>(kr);
             int cl = n0 + 16 * cc;
             cl = cl < p.n - 16 ? cl : p.n - 16;
-            b_voff[i] = (uint32_t)kr * (uint32_t)p.n + (uint32_t)cl;
+            v = (uint32_t)kr * (uint32_t)p.n + (uint32_t)cl;
+        } else if (I == C::A_COPIES + C::B_COPIES) {
+            int r = m0 + lane; r = r < p.lda - 1 ? r : p.lda - 1;
+            v = (uint32_t)r * 4u;
+        } else {
+            int x = nb0 + lane; x = x < p.nb - 1 ? x : p.nb - 1;
+            v = (uint32_t)x * 4u;
         }
-        if (wave == 2) { int r = m0 + lane; r = r < p.lda - 1 ? r : p.lda - 1; sc_voff = (uint32_t)r * 4u; }
-        if (wave == 3) { int x = nb0 + lane; x = x < p.nb - 1 ? x : p.nb - 1; sc_voff = (uint32_t)x * 4u; }
+        voff[q] = v;
     }
     const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
-    auto issue_block = [&](int blk) {      // all 7 copies of K block `blk` (relative to kb_begin)
+    auto issue_block = [&](int blk) {      // all copies of K block `blk` (relative to kb_begin)
         const uint32_t st = lds_base + (uint32_t)(blk % C::NSTAGE) * C::STAGE_BYTES;
         const uint32_t kb = (uint32_t)(kb_begin + blk);
         const uint32_t a_k = kb * (uint32_t)KBLK * (uint32_t)p.lda, b_k = kb * (uint32_t)KBLK * (uint32_t)p.n;
-        copy16_global_to_lds(a_rsrc, st + wave * 1024, a_voff, a_k + (uint32_t)(16 * wave) * (uint32_t)p.lda);
-        copy16_global_to_lds(a_rsrc, st + (4 + wave) * 1024, a_voff, a_k + (uint32_t)(16 * (4 + wave)) * (uint32_t)p.lda);
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-            copy16_global_to_lds(b_rsrc, st + C::A_BYTES + (4 * i + wave) * 1024, b_voff[i], b_k);
-        if (wave < 2) copy16_global_to_lds(b_rsrc, st + C::A_BYTES + (16 + wave) * 1024, b_voff[4], b_k);
-        else if (wave == 2) copy4_global_to_lds(as_rsrc, st + C::A_BYTES + C::B_BYTES, sc_voff, kb * (uint32_t)p.lda * 4u);
-        else copy4_global_to_lds(bs_rsrc, st + C::A_BYTES + C::B_BYTES + 256, sc_voff, kb * (uint32_t)p.nb * 4u);
+        for (int q = 0; q < C::COPIES; q++) {
+            const int I = 4 * q + wave;          // wave-uniform
+            if (I < C::A_COPIES) copy16_global_to_lds(a_rsrc, st + I * 1024, voff[q], a_k);
+            else if (I < C::A_COPIES + C::B_COPIES) copy16_global_to_lds(b_rsrc, st + C::A_BYTES + (I - C::A_COPIES) * 1024, voff[q], b_k);
+            else if (I == C::A_COPIES + C::B_COPIES) copy4_global_to_lds(as_rsrc, st + C::A_BYTES + C::B_BYTES, voff[q], kb * (uint32_t)p.lda * 4u);
+            else copy4_global_to_lds(bs_rsrc, st + C::A_BYTES + C::B_BYTES + 256, voff[q], kb * (uint32_t)p.nb * 4u);
+        }
     };
 
     // ---- LDS read addresses ----
     const int krow_lane = 8 * g + (i16 >> 1);
     const int swz_a = swz_of_krow<C::CPR_A>(krow_lane);
+    const int swz_b = C::SWZ_B ? swz_of_krow<C::CPR_B>(krow_lane) : 0;
     const int a_lane_off = krow_lane * C::BM + (i16 & 1) * 8;
     const int b_lane_off = C::A_BYTES + krow_lane * C::BN + (i16 & 1) * 8;
 
@@ -626,8 +647,7 @@ void gemm_skinny_kernel(const GemmArgs p) {
     for (int j = 0; j < nkb; j++) {
         // blocks issued after block j so far: up to NSTAGE-2; wait until only those are outstanding
         int ahead = (nkb - 1 < j + C::NSTAGE - 2 ? nkb - 1 : j + C::NSTAGE - 2) - j;
-        if (ahead >= 3) wait_vmcnt<3 * C::COPIES>();
-        else if (ahead == 2) wait_vmcnt<2 * C::COPIES>();
+        if (C::NSTAGE >= 4 && ahead >= 2) wait_vmcnt<(C::NSTAGE >= 4 ? 2 : 0) * C::COPIES>();
         else if (ahead == 1) wait_vmcnt<C::COPIES>();
         else wait_vmcnt<0>();
         __syncthreads();      // block j complete in LDS; everyone is done with the stage of block j-1
@@ -652,7 +672,7 @@ void gemm_skinny_kernel(const GemmArgs p) {
             const int u = wave + 4 * x;                 // wave-uniform
             if (u < C::CPR_B) {
                 v8i breg;
-                const unsigned char* q = sbase + b_lane_off + (u << 4);
+                const unsigned char* q = sbase + b_lane_off + ((u ^ swz_b) << 4);
 #pragma unroll
                 for (int jj = 0; jj < 4; jj++) {
                     v2i y = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_V2I(q + jj * 32 * C::BN));
@@ -825,6 +845,25 @@ static hipError_t launch_shape(const GemmArgs& a, int mode, hipStream_t stream) 
     return launch_tr<BM, BN, WM, WN, 0>(a, grid, stream);
 }
 
+template <int BN, int NSTAGE>
+static hipError_t launch_skinny(const GemmArgs& a, int mode, hipStream_t stream) {
+    if (mode == 2 || a.epi != 0) return hipErrorInvalidValue;
+    using C = SkinnyCfg<BN, NSTAGE>;
+    auto k0 = gemm_skinny_kernel<BN, NSTAGE, 0>;
+    auto k1 = gemm_skinny_kernel<BN, NSTAGE, 1>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void*)k0, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    int tiles = ((a.n + C::BN - 1) / C::BN) * a.split_k * ((a.m + C::BM - 1) / C::BM);
+    if (mode == 1) hipLaunchKernelGGL(k1, dim3(tiles), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
+    else hipLaunchKernelGGL(k0, dim3(tiles), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
+    return hipGetLastError();
+}
+
 hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t stream) {
     switch (variant) {
         case 1: {
@@ -836,23 +875,9 @@ hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t str
         case 3: return launch_shape<128, 128, 64, 64>(a, mode, stream);
         case 4: return launch_shape<64, 128, 32, 64>(a, mode, stream);
         case 5: return launch_shape<256, 128, 64, 64>(a, mode, stream);
-        case 6: {
-            if (mode == 2) return hipErrorInvalidValue;
-            using C = SkinnyCfg;
-            auto k0 = gemm_skinny_kernel<0>;
-            auto k1 = gemm_skinny_kernel<1>;
-            static bool attr_done = false;
-            if (!attr_done) {
-                hipError_t e = hipFuncSetAttribute((const void*)k0, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-                if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-                if (e != hipSuccess) return e;
-                attr_done = true;
-            }
-            int tiles = ((a.n + C::BN - 1) / C::BN) * a.split_k * ((a.m + C::BM - 1) / C::BM);
-            if (mode == 1) hipLaunchKernelGGL(k1, dim3(tiles), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
-            else hipLaunchKernelGGL(k0, dim3(tiles), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
-            return hipGetLastError();
-        }
+        case 6: return launch_skinny<144, 4>(a, mode, stream);
+        case 7: return launch_skinny<256, 3>(a, mode, stream);
+        case 8: return launch_skinny<288, 3>(a, mode, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -870,7 +895,9 @@ int variant_lds_bytes(int variant) {
         case 3: return TileCfg<128, 128, 64, 64, 0>::LDS_BYTES;
         case 4: return TileCfg<64, 128, 32, 64, 0>::LDS_BYTES;
         case 5: return TileCfg<256, 128, 64, 64, 0>::LDS_BYTES;
-        case 6: return SkinnyCfg::LDS_BYTES;
+        case 6: return SkinnyCfg<144, 4>::LDS_BYTES;
+        case 7: return SkinnyCfg<256, 3>::LDS_BYTES;
+        case 8: return SkinnyCfg<288, 3>::LDS_BYTES;
         default: return 0;
     }
 }

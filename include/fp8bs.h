@@ -49,7 +49,9 @@ enum {
     FP8BS_VARIANT_T64x128 = 4,    /* skinny-M: 64(m) x 128(n) tile, 4 waves, split-K         */
     FP8BS_VARIANT_T256x128 = 5,   /* 256(m) x 128(n) tile, 8 waves                           */
     FP8BS_VARIANT_SKINNY64x144 = 6, /* bandwidth-bound: 64(m) x 144(n) tile, 4-stage copy ring */
-    FP8BS_VARIANT_COUNT = 7
+    FP8BS_VARIANT_SKINNY64x256 = 7, /* same, 256-wide tile (whole 128-byte lines), 3 stages      */
+    FP8BS_VARIANT_SKINNY64x288 = 8, /* same, 288-wide tile, 3 stages                             */
+    FP8BS_VARIANT_COUNT = 9
 };
 
 /* What fp8bs_plan() decides for a shape. Replaces the exact-(m,n,k) if-ladder of the reference

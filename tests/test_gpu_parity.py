@@ -59,14 +59,14 @@ def test_config1_and_entry_point_contract(pkg, oracle, dev):
 
 def test_golden_fixture_bit_exact(pkg, golden_gemm, dev):
     cpu, expected, _ = golden_gemm
-    for variant in (0, 1, 3, 4, 6):       # planner's choice, generic, 128x128 tile, 64x128 tile, 64x144 ring
+    for variant in (0, 1, 3, 4, 6, 7, 8): # planner's choice, generic, 128x128 tile, 64x128 tile, the three ring kernels
         out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1 if variant else 0)
         assert torch.equal(out.cpu().view(torch.int16), expected.view(torch.int16)), "variant %d" % variant
     out = pkg.custom_kernel(_to(cpu, dev), variant=4, split_k=2)            # exact data: split-K is exact too
     assert torch.equal(out.cpu().view(torch.int16), expected.view(torch.int16))
 
 
-@pytest.mark.parametrize("variant,split_k", [(1, 1), (2, 1), (3, 1), (4, 1), (5, 1), (6, 1), (2, 2), (3, 3), (4, 4), (5, 8), (4, 7), (6, 2), (6, 8)])
+@pytest.mark.parametrize("variant,split_k", [(1, 1), (2, 1), (3, 1), (4, 1), (5, 1), (6, 1), (2, 2), (3, 3), (4, 4), (5, 8), (4, 7), (6, 2), (6, 8), (7, 1), (7, 2), (7, 3), (8, 1), (8, 4)])
 def test_every_variant_and_split_on_config1(pkg, oracle, dev, variant, split_k):
     cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0])
     out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=split_k)
@@ -82,7 +82,7 @@ def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
     out = pkg.custom_kernel(_to(cpu, dev))
     _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d" % (m, n, k))
     if m % 16 == 0 and n % 16 == 0:
-        for variant in (2, 3, 4, 5, 6):
+        for variant in (2, 3, 4, 5, 6, 7, 8):
             out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1)
             _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d" % (m, n, k, variant))
 
