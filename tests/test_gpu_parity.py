@@ -179,3 +179,58 @@ def test_grouped_full_size_sampled_rows(pkg, oracle, dev):
             rows += [lo, hi - 1] + (torch.randint(lo, hi, (6,), generator=g)).tolist()
     rows = torch.tensor(sorted(set(rows)))
     _check(oracle, out[rows.to(dev)], oracle.ref_grouped(cpu, rows=rows), "config 5 sampled rows")
+
+
+def test_special_codes(pkg, oracle, dev):
+    """-0, the largest codes (+-448), the smallest subnormals and NaN codes: a NaN in a row of A or B
+    poisons exactly the outputs that row takes part in, everything else stays within the bar."""
+    m, n, k = 64, 128, 256
+    cpu = list(pkg.inputs.make_dense(pkg.inputs.CONFIGS[3], m=m, n=n, k=k))
+    a = cpu[0].t().contiguous().view(torch.uint8)        # storage [k][m]
+    b = cpu[1].t().contiguous().view(torch.uint8)        # storage [k][n]
+    a[0, :8] = torch.tensor([0x80, 0x7E, 0xFE, 0x01, 0x81, 0x00, 0x7E, 0x08], dtype=torch.uint8)
+    b[1, :8] = torch.tensor([0x7E, 0xFE, 0x80, 0x01, 0x81, 0x7E, 0x7E, 0x00], dtype=torch.uint8)
+    a[5, 3] = 0x7F                                       # NaN in row 3 of A
+    b[130, 17] = 0xFF                                    # NaN in row 17 of B
+    cpu[0] = a.view(torch.float8_e4m3fn).t()
+    cpu[1] = b.view(torch.float8_e4m3fn).t()
+    ref = oracle.ref_kernel(tuple(cpu)).float()
+    for variant in (0, 1, 3, 4, 6):
+        out = pkg.custom_kernel(_to(tuple(cpu), dev), variant=variant, split_k=1 if variant else 0).cpu().float()
+        nan_ref = torch.isnan(ref)
+        assert nan_ref[3].all() and nan_ref[:, 17].all() and int(nan_ref.sum()) == n + m - 1
+        assert torch.equal(torch.isnan(out), nan_ref), "variant %d: NaN pattern differs" % variant
+        ok = ~nan_ref
+        err = (out[ok] - ref[ok]).abs()
+        assert bool((err <= ATOL + RTOL * ref[ok].abs()).all()), "variant %d" % variant
+
+
+def test_graph_capture_and_replay(pkg, oracle, dev):
+    """The library neither allocates nor synchronises, so a call can be captured into a HIP graph;
+    replays (with eager work and synchronisation in between) reproduce the eager result bit for bit,
+    for the single-kernel path and for the split-K path (two kernels, workspace)."""
+    for cfg_kw, kw in ((dict(m=256, n=512, k=1024), {}), (dict(m=64, n=2304, k=2048), {})):
+        cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[3], **cfg_kw)
+        data = _to(cpu, dev)
+        eager = pkg.custom_kernel(data, **kw).clone()
+        a2 = _to(pkg.inputs.make_dense(pkg.inputs.CONFIGS[2], **cfg_kw), dev)
+        eager2 = pkg.custom_kernel((a2[0], a2[1], a2[2], a2[3], torch.zeros_like(eager))).clone()
+        static = tuple(t.clone() for t in data)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            pkg.custom_kernel(static, **kw)                   # warm-up on the capture stream (workspace exists)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            pkg.custom_kernel(static, **kw)
+        for rep in range(3):
+            src, want = (data, eager) if rep % 2 == 0 else (a2, eager2)
+            for dst, s in zip(static[:4], src[:4]):
+                dst.copy_(s)
+            static[4].fill_(3.0)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static[4].view(torch.int16), want.view(torch.int16)), "replay %d" % rep
+            pkg.custom_kernel(data)                           # eager work between replays
+            torch.cuda.synchronize()
