@@ -73,7 +73,7 @@ def load() -> ctypes.CDLL:
     lib.fp8bs_gemm_silu_mul.restype = i32
     lib.fp8bs_gemm_silu_mul.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]
     lib.fp8bs_moe_combine.restype = i32
-    lib.fp8bs_moe_combine.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
+    lib.fp8bs_moe_combine.argtypes = [vp, i32, vp, vp, vp, i32, i32, i32, vp]
     lib.fp8bs_convert_fnuz_to_fn.restype = i32
     lib.fp8bs_convert_fnuz_to_fn.argtypes = [vp, vp, sz, vp]
     _lib = lib

@@ -155,7 +155,8 @@ void gemm_tr_kernel(const GemmArgs p) {
     int total_slots = 0;                      // grouped: m-tile slots that exist (from row_offsets)
     if (MODE == 2)
         for (int x = 0; x < p.num_experts; x++) {
-            const int lo = p.row_offsets[x], hi = p.row_offsets[x + 1];
+            int lo = p.row_offsets[x], hi = p.row_offsets[x + 1];
+            lo = lo < 0 ? 0 : lo; hi = hi > p.m ? p.m : hi;       // a malformed table must not reach beyond the matrix
             total_slots += (hi > lo) ? (hi - (lo & ~15) + BM - 1) / BM : 0;
         }
     auto pick_tile = [&](int it) -> Tile {
@@ -180,6 +181,7 @@ void gemm_tr_kernel(const GemmArgs p) {
             int acc_tiles = 0;
             for (int x = 0; x < p.num_experts; x++) {
                 int lo = p.row_offsets[x], hi = p.row_offsets[x + 1];
+                lo = lo < 0 ? 0 : lo; hi = hi > p.m ? p.m : hi;
                 int s = lo & ~15;
                 int nt = (hi > lo) ? (hi - s + BM - 1) / BM : 0;
                 if (!found && slot < acc_tiles + nt) {

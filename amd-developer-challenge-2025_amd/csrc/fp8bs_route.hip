@@ -223,17 +223,18 @@ void route_assign_kernel(const int32_t* __restrict__ top_idx, int tokens, int ex
 
 // out[t][d] = sum_j weights[t][j] * y[slot_of[t][j]][d], fp32 accumulation in the order j = 0..topk-1,
 // one rounding to bf16 (role of pack_output, 2-amd-moe/amd-moe-submission.py:239-301, which accumulates
-// in fp16).  One block per token, 8 columns (16 bytes) per thread and step; entries with slot -1 are skipped.
+// in fp16).  One block per token, 8 columns (16 bytes) per thread and step; entries whose slot is not a
+// row of y (-1 or beyond) are skipped.
 typedef int cv4i __attribute__((ext_vector_type(4)));
 __global__ __launch_bounds__(RB)
 void moe_combine_kernel(const uint16_t* __restrict__ y, const int32_t* __restrict__ slot_of, const float* __restrict__ weights,
-                        uint16_t* __restrict__ out, int topk, int d) {
+                        uint16_t* __restrict__ out, int rows, int topk, int d) {
     const int t = blockIdx.x;
     for (int c = threadIdx.x * 8; c < d; c += RB * 8) {
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         for (int j = 0; j < topk; j++) {
             const int slot = slot_of[(size_t)t * topk + j];
-            if (slot < 0) continue;
+            if (slot < 0 || slot >= rows) continue;
             const float w = weights[(size_t)t * topk + j];
             const cv4i v = *(const cv4i*)(y + (size_t)slot * d + c);
 #pragma unroll
@@ -301,12 +302,12 @@ extern "C" int fp8bs_moe_route(const int32_t* top_idx, int tokens, int experts, 
     return hipGetLastError() == hipSuccess ? FP8BS_OK : FP8BS_ERR_LAUNCH;
 }
 
-extern "C" int fp8bs_moe_combine(const void* y, const int32_t* slot_of, const float* weights, void* out,
+extern "C" int fp8bs_moe_combine(const void* y, int rows, const int32_t* slot_of, const float* weights, void* out,
                                  int tokens, int topk, int d, void* stream) {
-    if (tokens < 0 || topk <= 0 || d < 0 || (d % 8) != 0) return FP8BS_ERR_BAD_SHAPE;
+    if (tokens < 0 || rows < 0 || topk <= 0 || d < 0 || (d % 8) != 0) return FP8BS_ERR_BAD_SHAPE;
     if (tokens == 0 || d == 0) return FP8BS_OK;
     if (!y || !slot_of || !weights || !out) return FP8BS_ERR_NULL_POINTER;
     hipLaunchKernelGGL(fp8bs::moe_combine_kernel, dim3(tokens), dim3(fp8bs::RB), 0, (hipStream_t)stream,
-                       (const uint16_t*)y, slot_of, weights, (uint16_t*)out, topk, d);
+                       (const uint16_t*)y, slot_of, weights, (uint16_t*)out, rows, topk, d);
     return hipGetLastError() == hipSuccess ? FP8BS_OK : FP8BS_ERR_LAUNCH;
 }

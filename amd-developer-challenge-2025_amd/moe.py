@@ -96,6 +96,6 @@ def combine(y: torch.Tensor, slot_of: torch.Tensor, weights: torch.Tensor) -> to
     d = y.shape[1]
     out = torch.empty(t, d, dtype=torch.bfloat16, device=y.device)
     with torch.cuda.device(y.device):
-        _lib.check(_lib.load().fp8bs_moe_combine(y.data_ptr(), slot_of.data_ptr(), weights.data_ptr(), out.data_ptr(),
+        _lib.check(_lib.load().fp8bs_moe_combine(y.data_ptr(), y.shape[0], slot_of.data_ptr(), weights.data_ptr(), out.data_ptr(),
                                                  t, k, d, torch.cuda.current_stream().cuda_stream))
     return out

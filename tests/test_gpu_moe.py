@@ -138,3 +138,25 @@ def test_expert_ffn_chain(pkg, moe, quant, oracle, mo, ro, dev):
     _within(oracle, y.cpu(), y_r, "chain: down projection")
     out_r = mo.combine_ref(y.cpu(), torch.from_numpy(slot_r), torch.gather(scores, 1, torch.from_numpy(top_r).long()))
     _within(oracle, out.cpu(), out_r, "chain: combine")
+
+
+def test_out_of_range_tables_are_ignored(pkg, moe, dev):
+    """row offsets beyond the matrix and slots beyond y must not write or read outside the tensors"""
+    g = torch.Generator().manual_seed(9)
+    y = torch.randn(32, 64, generator=g).to(torch.bfloat16).to(dev)
+    slot = torch.tensor([[0, 31], [5, 32], [-7, 4], [1000000, 2]], dtype=torch.int32, device=dev)
+    w = torch.ones(4, 2, device=dev)
+    out = moe.combine(y, slot, w).float().cpu()
+    yf = y.float().cpu()
+    assert torch.allclose(out[0], (yf[0] + yf[31]).to(torch.bfloat16).float())
+    assert torch.equal(out[1], yf[5]) and torch.equal(out[2], yf[4]) and torch.equal(out[3], yf[2])
+    data = pkg.inputs.make_grouped(pkg.inputs.CONFIGS[4], tokens=64, n=256, k=128, experts=4, topk=2)
+    a, b, a_scale, b_scale, row_offsets, c = (t.to(dev) for t in data)
+    good = pkg.grouped_kernel((a, b, a_scale, b_scale, row_offsets, torch.zeros_like(c))).clone()
+    bad = row_offsets.clone()
+    bad[-1] = 10 ** 6                                          # last expert claims rows far beyond the matrix
+    guard = torch.full((c.shape[0] + 64, c.shape[1]), 5.0, dtype=torch.bfloat16, device=dev)
+    out = pkg.grouped_kernel((a, b, a_scale, b_scale, bad, guard[:c.shape[0]]))
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), good.view(torch.int16))
+    assert bool((guard[c.shape[0]:] == 5.0).all())
