@@ -502,7 +502,7 @@ void gemm_tr_kernel(const GemmArgs p) {
                 const int row = m0 + wave_m * WM + half * HALF_ROWS + r;
                 const int col = (EPI == 1 ? (n0 + wave_n * WN) / 2 : n0 + wave_n * WN) + chunk * 8;
                 if (row >= row_lo && row < row_hi && col < ldc)
-                    *(v4i*)(p.c + (size_t)row * ldc + col) = val;
+                    __builtin_nontemporal_store(val, (v4i*)(p.c + (size_t)row * ldc + col));   // written once, not read again here
             }
         }
     }
@@ -578,10 +578,8 @@ void gemm_skinny_kernel(const GemmArgs p) {
     const int nkb = kb_end - kb_begin;
     const int nb0 = n0 / 128;
 
-    __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, (uint32_t)p.k * (uint32_t)p.lda, 0x00020000);
-    __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.b, 0, (uint32_t)p.k * (uint32_t)p.n, 0x00020000);
-    __amdgpu_buffer_rsrc_t as_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.as, 0, (uint32_t)kbt * (uint32_t)p.lda * 4u, 0x00020000);
-    __amdgpu_buffer_rsrc_t bs_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.bs, 0, (uint32_t)kbt * (uint32_t)p.nb * 4u, 0x00020000);
+    const uint32_t a_bytes = (uint32_t)p.k * (uint32_t)p.lda, b_bytes = (uint32_t)p.k * (uint32_t)p.n;
+    const uint32_t as_bytes = (uint32_t)kbt * (uint32_t)p.lda * 4u, bs_bytes = (uint32_t)kbt * (uint32_t)p.nb * 4u;
 
     // ---- copy plan.  The one-KiB copies of a block are numbered I = 4q + wave, q = 0..COPIES-1:
     //      I < A_COPIES the A tile, then B_COPIES of the B tile (copy Ib fills B chunks 64*Ib ..), then the
@@ -616,9 +614,17 @@ void gemm_skinny_kernel(const GemmArgs p) {
         voff[q] = v;
     }
     const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
-    auto issue_block = [&](int blk) {      // all copies of K block `blk` (relative to kb_begin)
+    // All copies of K block `blk` (relative to kb_begin).  Beyond the last block the same number of
+    // copies is issued against empty buffers (every lane out of range: zeros land in a free stage and no
+    // memory is read), which keeps the count of outstanding copies per wave the same in every iteration.
+    auto issue_block = [&](int blk) {
         const uint32_t st = lds_base + (uint32_t)(blk % C::NSTAGE) * C::STAGE_BYTES;
-        const uint32_t kb = (uint32_t)(kb_begin + blk);
+        const bool live = blk < nkb;
+        const uint32_t kb = (uint32_t)(kb_begin + (live ? blk : 0));
+        __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, live ? a_bytes : 0u, 0x00020000);
+        __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.b, 0, live ? b_bytes : 0u, 0x00020000);
+        __amdgpu_buffer_rsrc_t as_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.as, 0, live ? as_bytes : 0u, 0x00020000);
+        __amdgpu_buffer_rsrc_t bs_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.bs, 0, live ? bs_bytes : 0u, 0x00020000);
         const uint32_t a_k = kb * (uint32_t)KBLK * (uint32_t)p.lda, b_k = kb * (uint32_t)KBLK * (uint32_t)p.n;
 #pragma unroll
         for (int q = 0; q < C::COPIES; q++) {
@@ -644,16 +650,13 @@ void gemm_skinny_kernel(const GemmArgs p) {
         for (int x = 0; x < C::NT_MAX; x++) acc[t][x] = (v4f){0.f, 0.f, 0.f, 0.f};
 
     // ---- prologue: NSTAGE-1 blocks in flight ----
-    for (int b = 0; b < C::NSTAGE - 1 && b < nkb; b++) issue_block(b);
+    for (int b = 0; b < C::NSTAGE - 1; b++) issue_block(b);
 
     for (int j = 0; j < nkb; j++) {
-        // blocks issued after block j so far: up to NSTAGE-2; wait until only those are outstanding
-        int ahead = (nkb - 1 < j + C::NSTAGE - 2 ? nkb - 1 : j + C::NSTAGE - 2) - j;
-        if (C::NSTAGE >= 4 && ahead >= 2) wait_vmcnt<(C::NSTAGE >= 4 ? 2 : 0) * C::COPIES>();
-        else if (ahead == 1) wait_vmcnt<C::COPIES>();
-        else wait_vmcnt<0>();
+        // the NSTAGE-2 blocks issued after block j may still be on their way
+        wait_vmcnt<(C::NSTAGE - 2) * C::COPIES>();
         __syncthreads();      // block j complete in LDS; everyone is done with the stage of block j-1
-        if (j + C::NSTAGE - 1 < nkb) issue_block(j + C::NSTAGE - 1);
+        issue_block(j + C::NSTAGE - 1);
 
         const unsigned char* sbase = lds + (j % C::NSTAGE) * C::STAGE_BYTES;
         const unsigned char* sc = sbase + C::A_BYTES + C::B_BYTES;
@@ -693,6 +696,8 @@ void gemm_skinny_kernel(const GemmArgs p) {
             }
         }
     }
+
+    wait_vmcnt<0>();          // the trailing empty copies still target this workgroup's LDS
 
     // ---- epilogue ----
 #pragma unroll
