@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(HERE, "libfp8bs.so")
 EXPORTS = (
     "fp8bs_version", "fp8bs_strerror", "fp8bs_plan", "fp8bs_workspace_bytes",
     "fp8bs_gemm", "fp8bs_gemm_ex", "fp8bs_gemm_grouped",
-    "fp8bs_quantize_a", "fp8bs_quantize_b",
+    "fp8bs_quantize_a", "fp8bs_quantize_b", "fp8bs_gather_a",
     "fp8bs_moe_topk", "fp8bs_moe_route_workspace_bytes", "fp8bs_moe_route",
     "fp8bs_gemm_silu_mul", "fp8bs_moe_combine", "fp8bs_convert_fnuz_to_fn",
 )
@@ -64,6 +64,8 @@ def load() -> ctypes.CDLL:
     lib.fp8bs_quantize_a.argtypes = [vp, i32, i64, vp, i32, vp, vp, i32, i32, vp]
     lib.fp8bs_quantize_b.restype = i32
     lib.fp8bs_quantize_b.argtypes = [vp, i32, i64, vp, vp, i32, i32, vp]
+    lib.fp8bs_gather_a.restype = i32
+    lib.fp8bs_gather_a.argtypes = [vp, vp, i32, vp, vp, vp, i32, i32, vp]
     lib.fp8bs_moe_topk.restype = i32
     lib.fp8bs_moe_topk.argtypes = [vp, i32, i32, i32, vp, vp]
     lib.fp8bs_moe_route_workspace_bytes.restype = sz

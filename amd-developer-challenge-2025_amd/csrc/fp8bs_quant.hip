@@ -265,6 +265,137 @@ void fnuz_to_fn_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ ds
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------------
+// Row gather of an already quantised activation matrix: out row i = source row row_map[i], bytes and
+// scales, in the K-major storage layout (a[kk * rows + i]).  With top-k routing every token appears
+// top-k times in the expert-contiguous order (2-amd-moe/3-amd-fp8-moe-hip-myhgemm.py:174-191 copies
+// rows the same way); quantising the tokens once and gathering bytes costs an eighth of the arithmetic
+// of quantising every copy.
+//
+// In this layout the gather runs along the contiguous dimension (one byte per row), so it goes through
+// LDS: a workgroup takes KC consecutive k rows of the source (KC * src_rows bytes), transposes them in
+// registers (v_perm_b32, 4x4 bytes) to token-major order - LDS slot of token t holds its KC bytes - and
+// then every lane produces four consecutive output rows: one LDS read of KC bytes per row, the
+// transpose back, and KC dword stores (a wave writes 256 contiguous bytes of one k row per store).
+// Slot of token t is (t % 4) * ceil(src_rows / 4) + t / 4, which makes the LDS writes of phase 1
+// contiguous across lanes.
+// ---------------------------------------------------------------------------------------------------
+struct GatherArgs {
+    const uint8_t* src;       // [k][src_rows]
+    const float* src_scale;   // [k/128][src_rows]
+    const int32_t* row_map;   // [rows]
+    uint8_t* dst;             // [k][rows]
+    float* dst_scale;         // [k/128][rows]
+    int rows, k, src_rows;
+    int rows_per_wg;          // multiple of 4
+};
+
+// rw[r] = bytes (c0..c3) of line r  ->  out[j] = bytes (line0..line3) of column j
+__device__ __forceinline__ void transpose4x4(const uint32_t rw[4], uint32_t out[4]) {
+    const uint32_t lo01 = __builtin_amdgcn_perm(rw[1], rw[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(rw[1], rw[0], 0x07030602u);
+    const uint32_t lo23 = __builtin_amdgcn_perm(rw[3], rw[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(rw[3], rw[2], 0x07030602u);
+    out[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u); out[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+    out[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u); out[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+}
+
+template <int KC>
+__global__ __launch_bounds__(256)
+void gather_a_kernel(const GatherArgs p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char slots[];     // [4 * quarter][KC]
+    constexpr int KG = KC / 4;
+    const int tid = threadIdx.x;
+    const int k0 = blockIdx.x * KC;
+    const int quarter = (p.src_rows + 3) / 4;
+    // ---- phase 1: KC source rows -> token-major slots ----
+    __amdgpu_buffer_rsrc_t src_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.src, 0, (uint32_t)p.k * (uint32_t)p.src_rows, 0x00020000);
+    for (int task = tid; task < quarter; task += 256) {
+        uint32_t tok[4][KG];                       // tok[j][kg]: bytes (k rows 4kg..4kg+3) of token 4*task + j
+#pragma unroll
+        for (int kg = 0; kg < KG; kg++) {
+            uint32_t rw[4], c[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                rw[r] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(src_rsrc, (uint32_t)(k0 + 4 * kg + r) * (uint32_t)p.src_rows + 4u * (uint32_t)task, 0, 0);
+            transpose4x4(rw, c);
+#pragma unroll
+            for (int j = 0; j < 4; j++) tok[j][kg] = c[j];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            unsigned char* d = slots + (size_t)(j * quarter + task) * KC;
+#pragma unroll
+            for (int kg = 0; kg < KG; kg++) *(uint32_t*)(d + 4 * kg) = tok[j][kg];
+        }
+    }
+    __syncthreads();
+    // ---- phase 2: four consecutive output rows per lane ----
+    const int row_begin = blockIdx.y * p.rows_per_wg;
+    int row_end = row_begin + p.rows_per_wg;
+    row_end = row_end < p.rows ? row_end : p.rows;
+    for (int i0 = row_begin + 4 * tid; i0 < row_end; i0 += 1024) {
+        const v4i map = *(const v4i*)(p.row_map + i0);
+        uint32_t tok[4][KG];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t t = (uint32_t)map[j];
+            const bool ok = t < (uint32_t)p.src_rows;
+            const unsigned char* sp = slots + (size_t)((t & 3u) * (uint32_t)quarter + (t >> 2)) * KC;
+#pragma unroll
+            for (int kg = 0; kg < KG; kg++) tok[j][kg] = ok ? *(const uint32_t*)(sp + 4 * kg) : 0u;
+        }
+#pragma unroll
+        for (int kg = 0; kg < KG; kg++) {
+            uint32_t rw[4], c[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) rw[j] = tok[j][kg];
+            transpose4x4(rw, c);                   // c[r] = bytes (rows i0..i0+3) of k row 4kg + r
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                __builtin_nontemporal_store(c[r], (uint32_t*)(p.dst + (size_t)(k0 + 4 * kg + r) * (size_t)p.rows + i0));
+        }
+        // the scales of a K block travel with its first k rows
+        if ((k0 & 127) == 0) {
+            v4f sc;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t t = (uint32_t)map[j];
+                sc[j] = t < (uint32_t)p.src_rows ? p.src_scale[(size_t)(k0 >> 7) * p.src_rows + t] : 1e-12f;
+            }
+            *(v4f*)(p.dst_scale + (size_t)(k0 >> 7) * p.rows + i0) = sc;
+        }
+    }
+}
+
+// any alignment, any size: one output byte per thread
+__global__ __launch_bounds__(256)
+void gather_a_bytes_kernel(const GatherArgs p) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= p.rows) return;
+    const uint32_t t = (uint32_t)p.row_map[i];
+    const bool ok = t < (uint32_t)p.src_rows;
+    for (int kk = blockIdx.y; kk < p.k; kk += gridDim.y) {
+        p.dst[(size_t)kk * p.rows + i] = ok ? p.src[(size_t)kk * p.src_rows + t] : (uint8_t)0;
+        if ((kk & 127) == 0) p.dst_scale[(size_t)(kk >> 7) * p.rows + i] = ok ? p.src_scale[(size_t)(kk >> 7) * p.src_rows + t] : 1e-12f;
+    }
+}
+
+template <int KC>
+static hipError_t launch_gather(const GatherArgs& a, hipStream_t stream) {
+    const int quarter = (a.src_rows + 3) / 4;
+    const int lds = 4 * quarter * KC;
+    auto kern = gather_a_kernel<KC>;
+    static int attr_lds = 0;     // largest dynamic-LDS size allowed so far; raising it again is harmless
+    if (lds > 65536 && lds > attr_lds) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        attr_lds = lds;
+    }
+    dim3 grid((unsigned)(a.k / KC), (unsigned)((a.rows + a.rows_per_wg - 1) / a.rows_per_wg));
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
+    return hipGetLastError();
+}
+
 }  // namespace fp8bs
 
 extern "C" int fp8bs_convert_fnuz_to_fn(const void* src, void* dst, size_t nbytes, void* stream) {
@@ -306,4 +437,27 @@ extern "C" int fp8bs_quantize_a(const void* x, int x_dtype, int64_t ldx, const i
 
 extern "C" int fp8bs_quantize_b(const void* w, int w_dtype, int64_t ldw, void* b, float* b_scale, int n, int k, void* stream) {
     return quantize_common(w, w_dtype, ldw, nullptr, 0, b, b_scale, n, k, true, stream);
+}
+
+extern "C" int fp8bs_gather_a(const void* a_src, const float* a_scale_src, int src_rows, const int32_t* row_map,
+                              void* a, float* a_scale, int m, int k, void* stream) {
+    if (m < 0 || k < 0 || src_rows < 0 || (k % 128) != 0) return FP8BS_ERR_BAD_SHAPE;
+    if (m == 0 || k == 0) return FP8BS_OK;
+    if (!row_map || !a || !a_scale || (src_rows > 0 && (!a_src || !a_scale_src))) return FP8BS_ERR_NULL_POINTER;
+    if ((size_t)src_rows * (size_t)k > 0xFFFFFFFFull) return FP8BS_ERR_TOO_LARGE;       // buffer addressing
+    fp8bs::GatherArgs g{(const uint8_t*)a_src, a_scale_src, row_map, (uint8_t*)a, a_scale, m, k, src_rows, 8192};
+    hipStream_t s = (hipStream_t)stream;
+    // dword loads of source rows, dword stores of output rows, 16-byte loads of the map and stores of
+    // the scales: everything must sit on those boundaries, and the KC source rows must fit the LDS
+    const bool aligned = (src_rows % 4) == 0 && (m % 4) == 0 && src_rows > 0 &&
+                         ((((uintptr_t)a_src | (uintptr_t)a) & 3) == 0) && ((((uintptr_t)row_map | (uintptr_t)a_scale) & 15) == 0);
+    hipError_t e;
+    if (aligned && src_rows <= 4096) e = fp8bs::launch_gather<16>(g, s);
+    else if (aligned && src_rows <= 8192) e = fp8bs::launch_gather<8>(g, s);
+    else if (aligned && src_rows <= 40960) e = fp8bs::launch_gather<4>(g, s);
+    else {
+        hipLaunchKernelGGL(fp8bs::gather_a_bytes_kernel, dim3((unsigned)((m + 255) / 256), (unsigned)(k < 4096 ? k : 4096)), dim3(256), 0, s, g);
+        e = hipGetLastError();
+    }
+    return e == hipSuccess ? FP8BS_OK : FP8BS_ERR_LAUNCH;
 }

@@ -1,7 +1,7 @@
 """GPU block quantisers: row-major fp32/bf16 matrices -> the operands ``custom_kernel`` takes.
 
 The reference has no quantiser (its operands arrive quantised, 1-amd-fp8-mm/0-amd-fp8-mm-new-begins.py:66-77);
-these wrap ``fp8bs_quantize_a`` / ``fp8bs_quantize_b`` of libfp8bs.so and return tensors with exactly
+these wrap ``fp8bs_quantize_a`` / ``fp8bs_quantize_b`` / ``fp8bs_gather_a`` of libfp8bs.so and return tensors with exactly
 the shapes, dtypes and K-major strides of that contract.  The rule is the one of ``inputs.quantize_a`` /
 ``inputs.quantize_b`` (the host-side quantisers), bit for bit.  No fallback: without the library the
 import of ``_lib`` raises.
@@ -64,3 +64,30 @@ def quantize_b(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
             w.data_ptr(), _DTYPES[w.dtype], w.stride(0) if n > 1 else max(k, 1),
             b_store.data_ptr(), s_store.data_ptr(), n, k, stream))
     return b_store.t(), s_store.t()
+
+
+def gather_a(a: torch.Tensor, a_scale: torch.Tensor, row_map: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Rows ``row_map`` of quantised activations: (a [T, K], a_scale [T, K/128]) K-major -> the same for M rows.
+
+    ``gather_a(*quantize_a(x), row_map)`` returns exactly what ``quantize_a(x, row_map)`` returns, but
+    quantises every token once instead of once per routed copy (the reference copies rows into expert
+    order, 2-amd-moe/3-amd-fp8-moe-hip-myhgemm.py:174-191).  Entries of ``row_map`` outside [0, T) give
+    zero rows with scale 1e-12.
+    """
+    if a.dtype != torch.float8_e4m3fn or a_scale.dtype != torch.float32 or a.dim() != 2 or a_scale.dim() != 2 or not a.is_cuda:
+        raise TypeError("a must be a float8_e4m3fn and a_scale a float32 2-D tensor on the GPU")
+    t, k = a.shape
+    if k % 128 != 0 or tuple(a_scale.shape) != (t, k // 128):
+        raise ValueError("a [T, K] needs K %% 128 == 0 and a_scale [T, K/128]; got %s and %s" % (tuple(a.shape), tuple(a_scale.shape)))
+    if not a.t().is_contiguous() or not a_scale.t().is_contiguous():
+        raise ValueError("a and a_scale must be K-major (stride 1 along rows)")
+    if row_map.dtype != torch.int32 or row_map.dim() != 1 or row_map.device != a.device or not row_map.is_contiguous():
+        raise ValueError("row_map must be a contiguous int32 vector on a's device")
+    m = row_map.numel()
+    a_store = torch.empty(k, m, dtype=torch.float8_e4m3fn, device=a.device)
+    s_store = torch.empty(k // 128, m, dtype=torch.float32, device=a.device)
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.load().fp8bs_gather_a(a.data_ptr(), a_scale.data_ptr(), t, row_map.data_ptr(),
+                                              a_store.data_ptr(), s_store.data_ptr(), m, k,
+                                              torch.cuda.current_stream().cuda_stream))
+    return a_store.t(), s_store.t()

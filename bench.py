@@ -220,6 +220,13 @@ def main():
         per_config["quant_a_gather_fp32_4096to32768x7168"] = {
             "us": round(us, 2), "us_min": round(us_min, 2), "gbs": round(by / us * 1e-3, 1), "bytes": by, "bound": "hbm",
             "frac": round(by / us * 1e-3 / PEAK_HBM_GBS, 4), "note": "token rows read once algorithmically, written 8 times"}
+        # the same operand by quantising every token once and gathering bytes: two kernels
+        us, us_min = time_calls(lambda i: quant.gather_a(*quant.quantize_a(x), row_map), max(args.steps // 2, 5), 3)
+        by2 = by + 2 * (cfg5.m * cfg5.k + 4 * cfg5.m * (cfg5.k // 128))
+        per_config["quant_a_then_gather_fp32_4096to32768x7168"] = {
+            "us": round(us, 2), "us_min": round(us_min, 2), "gbs": round(by2 / us * 1e-3, 1), "bytes": by2, "bound": "hbm",
+            "frac": round(by2 / us * 1e-3 / PEAK_HBM_GBS, 4),
+            "note": "quantise 4096 rows (fp32 in, fp8 out), then gather 32768 rows of bytes and scales"}
         x = row_map = scores = None
         # expert FFN of configuration 5: gate/up GEMM with the fused silu-mul epilogue (N = 2 x 2048
         # interleaved), quantisation of h, down projection (N = 7168, K = 2048), weighted un-permute

@@ -124,6 +124,17 @@ enum { FP8BS_DTYPE_F32 = 0, FP8BS_DTYPE_BF16 = 1 };
 int fp8bs_quantize_a(const void* x, int x_dtype, int64_t ldx, const int32_t* row_map, int src_rows,
                      void* a, float* a_scale, int m, int k, void* stream);
 
+/* Row gather of quantised activations: a[kk][i] = a_src[kk][row_map[i]] and a_scale[kb][i] =
+ * a_scale_src[kb][row_map[i]] for i < m (a_src: K rows of src_rows bytes, a_scale_src: K/128 rows of
+ * src_rows floats; entries of row_map outside [0, src_rows) give zero bytes and the scale 1e-12, what
+ * fp8bs_quantize_a writes for a zero row).  Quantising the tokens once and gathering gives the same
+ * bytes as fp8bs_quantize_a with the same row_map at an eighth of the arithmetic when every token is
+ * routed to 8 experts; the reference copies rows into expert order the same way
+ * (2-amd-moe/3-amd-fp8-moe-hip-myhgemm.py:174-191).  Fast path: src_rows and m multiples of 4,
+ * src_rows <= 40960, row_map and a_scale 16-byte aligned; anything else takes a byte-wise kernel. */
+int fp8bs_gather_a(const void* a_src, const float* a_scale_src, int src_rows, const int32_t* row_map,
+                   void* a, float* a_scale, int m, int k, void* stream);
+
 /* Weights: w [n][k] -> b (K rows of n bytes) and b_scale (K/128 rows of ceil(n/128) floats), one scale
  * per 128x128 block; a partial last block of rows takes its maximum over the rows that exist. */
 int fp8bs_quantize_b(const void* w, int w_dtype, int64_t ldw, void* b, float* b_scale, int n, int k,

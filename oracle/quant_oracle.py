@@ -26,6 +26,9 @@ How each function is pinned (tests/test_quant_oracle.py):
                     invariants: |decoded q| <= 448, the largest |x| of every non-zero block maps to
                     code 448, relative error of normal values <= 2^-4, re-quantising the dequantised
                     values returns the same codes
+  * gather_a_ref    defined by the identity it is checked against: gather_a_ref(quantize_a_ref(x), map) must
+                    equal quantize_a_ref(x, map) bit for bit (a block's scale and bytes depend on its own row
+                    only), including out-of-range entries; plus a hand-written 3-row case
   * fnuz_to_fn_ref  (e4m3fnuz, the reference's gfx942 type, 1-amd-fp8-mm/amd-fp8-mm-submission.py:20-21:
                     bias 8, NaN 0x80, no -0)  torch's own float8_e4m3fnuz -> float32 -> float8_e4m3fn
                     casts on all 256 codes
@@ -88,6 +91,24 @@ def quantize_a_ref(x: np.ndarray, row_map=None):
     q = np.clip(xb / scale[:, :, None], -FP8_MAX, FP8_MAX).astype(np.float32)
     codes = encode_e4m3fn(q.reshape(m, k))
     return np.ascontiguousarray(codes.T), np.ascontiguousarray(scale.T)
+
+
+def gather_a_ref(q: np.ndarray, scale: np.ndarray, row_map) -> tuple:
+    """Storage-order q uint8 [K][T], scale float32 [K/128][T] -> the same for rows row_map (int [M]).
+
+    Entries of row_map outside [0, T) give zero bytes and the scale 1e-12 (a zero row quantised).
+    Row copy into expert order: 2-amd-moe/3-amd-fp8-moe-hip-myhgemm.py:174-191.
+    """
+    q = np.asarray(q, dtype=np.uint8)
+    scale = np.asarray(scale, dtype=np.float32)
+    row_map = np.asarray(row_map, dtype=np.int64)
+    ok = (row_map >= 0) & (row_map < q.shape[1])
+    safe = np.where(ok, row_map, 0)
+    if q.shape[1] == 0:
+        return np.zeros((q.shape[0], row_map.size), np.uint8), np.full((scale.shape[0], row_map.size), TINY, np.float32)
+    out_q = np.where(ok[None, :], q[:, safe], np.uint8(0)).astype(np.uint8)
+    out_s = np.where(ok[None, :], scale[:, safe], TINY).astype(np.float32)
+    return np.ascontiguousarray(out_q), np.ascontiguousarray(out_s)
 
 
 def quantize_b_ref(w: np.ndarray):

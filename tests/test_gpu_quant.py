@@ -102,6 +102,51 @@ def test_quantize_a_row_map(quant, qo, dev):
     assert np.array_equal(s, ws) and np.array_equal(q, wq)
 
 
+@pytest.mark.parametrize("tokens,rows,k", [(64, 256, 128),          # 16 k rows per workgroup
+                                           (4096, 8192 + 4, 256),   # two row chunks, the second 4 rows
+                                           (4100, 512, 128),        # 8 k rows per workgroup
+                                           (8200, 256, 128),        # 4 k rows per workgroup
+                                           (50, 180, 256),          # tokens not a multiple of 4: byte-wise kernel
+                                           (64, 90, 128),           # rows not a multiple of 4: byte-wise kernel
+                                           (4, 4, 128)])
+def test_gather_a_bit_exact(quant, qo, dev, tokens, rows, k):
+    g = torch.Generator().manual_seed(tokens * 7 + rows)
+    q_src = torch.randint(0, 256, (k, tokens), dtype=torch.uint8, generator=g)
+    s_src = torch.rand(k // 128, tokens, generator=g) + 0.01
+    row_map = torch.randint(0, tokens, (rows,), dtype=torch.int32, generator=g)
+    row_map[::17] = -1
+    row_map[3::29] = tokens
+    row_map[-1] = tokens - 1
+    a = q_src.to(dev).view(torch.float8_e4m3fn).t()
+    q, s = _store(*quant.gather_a(a, s_src.to(dev).t(), row_map.to(dev)))
+    wq, ws = qo.gather_a_ref(q_src.numpy(), s_src.numpy(), row_map.numpy())
+    assert q.shape == (k, rows) and s.shape == (k // 128, rows)
+    assert np.array_equal(q, wq) and np.array_equal(s, ws)
+
+
+def test_gather_after_quantise_equals_fused_gather(quant, dev):
+    """Full MoE size: 4096 tokens routed 8 ways, K = 7168; both routes to the same 32768-row operand."""
+    g = torch.Generator().manual_seed(77)
+    x = (torch.randn(4096, 7168, generator=g) * 3).to(dev)
+    row_map = torch.randint(0, 4096, (32768,), dtype=torch.int32, generator=g).to(dev)
+    a1, s1 = quant.quantize_a(x, row_map)
+    a2, s2 = quant.gather_a(*quant.quantize_a(x), row_map)
+    assert a2.shape == a1.shape and a2.stride() == a1.stride() and s2.stride() == s1.stride()
+    assert torch.equal(a1.view(torch.uint8), a2.view(torch.uint8)) and torch.equal(s1, s2)
+
+
+def test_gather_a_argument_errors(quant, dev):
+    a, s = quant.quantize_a(torch.randn(8, 128, device=dev))
+    with pytest.raises(ValueError):
+        quant.gather_a(a, s, torch.zeros(4, dtype=torch.int64, device=dev))
+    with pytest.raises(ValueError):
+        quant.gather_a(a, s[:, :0], torch.zeros(4, dtype=torch.int32, device=dev))
+    with pytest.raises(TypeError):
+        quant.gather_a(a.view(torch.uint8), s, torch.zeros(4, dtype=torch.int32, device=dev))
+    q0, s0 = quant.gather_a(a, s, torch.zeros(0, dtype=torch.int32, device=dev))
+    assert q0.shape == (0, 128) and s0.shape == (0, 1)
+
+
 @pytest.mark.parametrize("n,k,dtype", [(256, 256, torch.float32), (2112, 512, torch.float32), (200, 256, torch.float32),
                                        (384, 384, torch.bfloat16)])
 def test_quantize_b_bit_exact(quant, qo, dev, n, k, dtype):

@@ -115,6 +115,27 @@ def test_row_map_gathers_rows(qo):
             assert not q[:, i].any() and s[0, i] == np.float32(1e-12)
 
 
+def test_gather_of_quantised_rows_equals_quantising_gathered_rows(qo):
+    rng = np.random.default_rng(15)
+    x = (rng.standard_normal((37, 384)) * rng.choice([1e-3, 1.0, 50.0], size=(37, 1))).astype(np.float32)
+    x[5] = 0
+    row_map = np.concatenate([rng.integers(0, 37, size=90), [-1, 37, 1000, -5, 0, 36]])
+    rng.shuffle(row_map)
+    want_q, want_s = qo.quantize_a_ref(x, row_map)
+    got_q, got_s = qo.gather_a_ref(*qo.quantize_a_ref(x), row_map)
+    assert got_q.shape == want_q.shape == (384, 96) and got_s.shape == want_s.shape == (3, 96)
+    assert np.array_equal(got_q, want_q) and np.array_equal(got_s, want_s)
+    # by hand: three rows, one K block
+    q = np.arange(3 * 128, dtype=np.uint8).reshape(128, 3)
+    sc = np.array([[0.5, 2.0, 8.0]], dtype=np.float32)
+    gq, gs = qo.gather_a_ref(q, sc, [2, 0, 3, 2])
+    assert np.array_equal(gq[:, 0], q[:, 2]) and np.array_equal(gq[:, 1], q[:, 0]) and not gq[:, 2].any() and np.array_equal(gq[:, 3], q[:, 2])
+    assert gs.tolist() == [[8.0, 0.5, float(np.float32(1e-12)), 8.0]]
+    # no source rows at all: every entry is out of range
+    eq, es = qo.gather_a_ref(np.zeros((128, 0), np.uint8), np.zeros((1, 0), np.float32), [0, 1])
+    assert eq.shape == (128, 2) and not eq.any() and (es == np.float32(1e-12)).all()
+
+
 def test_fnuz_to_fn_against_torch_casts(qo):
     codes = np.arange(256, dtype=np.uint8)
     vals = torch.from_numpy(codes.copy()).view(torch.float8_e4m3fnuz).float()
