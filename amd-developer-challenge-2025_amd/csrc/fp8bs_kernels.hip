@@ -140,7 +140,11 @@ void gemm_tr_kernel(const GemmArgs p) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 4, i16 = lane & 15;
-    const int wave_m = wave % C::WAVES_M, wave_n = wave / C::WAVES_M;
+    // Waves w and w+4 share a SIMD.  With 4 x 2 waves they get m positions two apart, so that in a tile
+    // whose valid rows end at half height (the last tile of an expert, of M) every SIMD keeps one wave
+    // with work instead of two SIMDs keeping both.
+    const int wave_n = wave / C::WAVES_M;
+    const int wave_m = (C::WAVES_M == 4 && C::NWAVES == 8) ? ((wave + 2 * wave_n) & 3) : wave % C::WAVES_M;
 
     // ---- tiles ---------------------------------------------------------------------------------
     // The workgroup is persistent: it walks the tiles  blockIdx.x, blockIdx.x + gridDim.x, ...  and
@@ -332,6 +336,8 @@ void gemm_tr_kernel(const GemmArgs p) {
     // one 128-block), loaded straight from memory two k blocks ahead.
     int nblk = (n0 + wave_n * WN) / 128;
     nblk = __builtin_amdgcn_readfirstlane(nblk < p.nb - 1 ? nblk : p.nb - 1);
+    // does any row of this wave's tile get stored?
+    const bool wave_active = __builtin_amdgcn_readfirstlane((m0 + wave_m * WM < row_hi && m0 + wave_m * WM + WM > row_lo) ? 1 : 0) != 0;
 
     v4f acc[C::MT][C::NT];
 #pragma unroll
@@ -367,9 +373,11 @@ void gemm_tr_kernel(const GemmArgs p) {
         }
 
         v8i areg[C::MT], breg[2];
+        if (wave_active) {
 #pragma unroll
-        for (int t = 0; t < C::MT; t++) read_a(areg[t], t, lds);
-        read_b(breg[0], 0, lds);
+            for (int t = 0; t < C::MT; t++) read_a(areg[t], t, lds);
+            read_b(breg[0], 0, lds);
+        }
 
         // One K block (index j, in stage j&1).  The flags are compile-time so that the step sequence
         // is one straight-line block for the instruction scheduler.
@@ -377,6 +385,23 @@ void gemm_tr_kernel(const GemmArgs p) {
             constexpr bool HAS_NEXT = decltype(has_next_tag)::value;      // block j+1 exists
             constexpr bool HAS_NEXT2 = decltype(has_next2_tag)::value;    // block j+2 exists
             const int cur_stage = j & 1;
+            if (!wave_active) {
+                // none of this wave's rows is stored: it only does its share of the copies, in the
+                // same order and around the same single barrier as the waves that compute
+                if constexpr (HAS_NEXT) {
+                    [&]<int... Q>(std::integer_sequence<int, Q...>) {
+                        (issue_one(cp, cur_stage ^ 1, j + 1, std::integral_constant<int, NL_LATE + Q>{}), ...);
+                    }(std::make_integer_sequence<int, NL_EARLY>{});
+                }
+                __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
+                __syncthreads();
+                if constexpr (HAS_NEXT2) {
+                    [&]<int... Q>(std::integer_sequence<int, Q...>) {
+                        (issue_one(cp, cur_stage, j + 2, std::integral_constant<int, Q>{}), ...);
+                    }(std::make_integer_sequence<int, NL_LATE>{});
+                }
+                return;
+            }
             const unsigned char* sbase = lds + cur_stage * C::STAGE_BYTES;
             const unsigned char* snext = lds + (cur_stage ^ 1) * C::STAGE_BYTES;
             float sc[C::MT];
@@ -441,8 +466,9 @@ void gemm_tr_kernel(const GemmArgs p) {
         if (nxt.kb_end > nxt.kb_begin) { issue_all(ncp, 0, 0); prefetched = true; }
     }
 
-    // ---- epilogue -----------------------------------------------------------------------------
-    if (MODE == 1) {
+    // ---- epilogue (a wave without valid rows has nothing to store; no barrier in here) -----------
+    if (!wave_active) {
+    } else if (MODE == 1) {
         // split-K: fp32 partial tile, 16 bytes per lane
 #pragma unroll
         for (int t = 0; t < C::MT; t++) {
