@@ -54,6 +54,11 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 // 16 bytes per lane, global -> LDS without passing through registers (buffer_load_dwordx4 ... lds):
 // lane l's bytes land at lds_base + 16*l; lds_base and wave_offset must be wave-uniform (SGPRs), the
 // address is buffer base + lane_offset + wave_offset.
+// M0 (the LDS base of such a load) is written inside the statement.  The compiler reserves M0 and warns
+// when it sees it among the clobbers; nothing it generates for these kernels reads M0 (LDS instructions
+// need no M0 on gfx9, and there are no indirect register moves, GWS or message instructions here).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void copy16_global_to_lds(__amdgpu_buffer_rsrc_t rsrc, uint32_t lds_base, uint32_t lane_offset, uint32_t wave_offset) {
     asm volatile("s_mov_b32 m0, %2\n\tbuffer_load_dwordx4 %0, %1, %3 offen lds"
                  :: "v"(lane_offset), "s"(rsrc), "s"(lds_base), "s"(wave_offset) : "memory", "m0");
@@ -63,6 +68,7 @@ __device__ __forceinline__ void copy4_global_to_lds(__amdgpu_buffer_rsrc_t rsrc,
     asm volatile("s_mov_b32 m0, %2\n\tbuffer_load_dword %0, %1, %3 offen lds"
                  :: "v"(lane_offset), "s"(rsrc), "s"(lds_base), "s"(wave_offset) : "memory", "m0");
 }
+#pragma clang diagnostic pop
 
 // ---------------------------------------------------------------------------------------------------
 // Tile -> workgroup mapping.  Workgroups are dealt round-robin to the 8 XCDs (each with its own L2),
@@ -118,7 +124,8 @@ struct TileCfg {
 template <int CPR>
 __device__ __forceinline__ int swz_of_krow(int krow) {
     // rows per 256-byte bank sweep = 16/CPR; consecutive sweeps get consecutive XOR masks
-    return (krow / (16 / CPR)) % CPR;
+    constexpr int ROWS_PER_SWEEP = CPR <= 16 ? 16 / CPR : 1;      // (wider rows are never swizzled)
+    return (krow / ROWS_PER_SWEEP) % CPR;
 }
 
 // EPI 0: plain bf16 output.  EPI 1: gate/up pairs - column 2i is gate_i, column 2i+1 is up_i - are

@@ -207,17 +207,18 @@ void route_assign_kernel(const int32_t* __restrict__ top_idx, int tokens, int ex
     if (t >= tokens) return;
 #pragma unroll
     for (int j = 0; j < MAX_TOPK; j++) {
-        if (j >= topk) break;
-        int dest = -1;
-        if (ch[j] >= 0) {
-            const uint32_t* bm = bits + ch[j] * (RB / 32);
-            int rank = __builtin_popcount(bm[w] & ((1u << bit) - 1u));
+        if (j < topk) {
+            int dest = -1;
+            if (ch[j] >= 0) {
+                const uint32_t* bm = bits + ch[j] * (RB / 32);
+                int rank = __builtin_popcount(bm[w] & ((1u << bit) - 1u));
 #pragma unroll
-            for (int x = 0; x < RB / 32; x++) rank += x < w ? __builtin_popcount(bm[x]) : 0;
-            dest = first_row[ch[j]] + rank;
-            row_map[dest] = t;
+                for (int x = 0; x < RB / 32; x++) rank += x < w ? __builtin_popcount(bm[x]) : 0;
+                dest = first_row[ch[j]] + rank;
+                row_map[dest] = t;
+            }
+            if (slot_of) slot_of[(size_t)t * topk + j] = dest;
         }
-        if (slot_of) slot_of[(size_t)t * topk + j] = dest;
     }
 }
 
