@@ -125,7 +125,15 @@ int check_common(const void* a, const void* b, const float* as, const float* bs,
         return FP8BS_ERR_NULL_POINTER;
     }
     if ((uint64_t)m * (uint64_t)k >= (1ull << 32) || (uint64_t)n * (uint64_t)k >= (1ull << 32)) return FP8BS_ERR_TOO_LARGE;
+    if ((((uintptr_t)as | (uintptr_t)bs) & 3) != 0 || ((uintptr_t)c & 1) != 0) return FP8BS_ERR_BAD_SHAPE;   // element alignment
     return FP8BS_OK;
+}
+
+// The tiled and streaming kernels copy and store 16 bytes at a time: operands, output and workspace
+// must start on 16-byte boundaries (rows then do too, because m and n are multiples of 16 there).
+// Anything else is left to the generic kernel, which accesses single elements.
+bool vector_aligned(const void* a, const void* b, const void* c, const void* ws) {
+    return ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)ws) & 15) == 0);
 }
 
 }  // namespace
@@ -138,7 +146,7 @@ const char* fp8bs_strerror(int status) {
     switch (status) {
         case FP8BS_OK: return "success";
         case FP8BS_ERR_NULL_POINTER: return "a required pointer is NULL";
-        case FP8BS_ERR_BAD_SHAPE: return "bad shape: m, n, k must be non-negative and k a multiple of 128";
+        case FP8BS_ERR_BAD_SHAPE: return "bad shape: m, n, k must be non-negative and k a multiple of 128 (or a pointer is not aligned to its element type)";
         case FP8BS_ERR_WORKSPACE: return "workspace missing or smaller than fp8bs_workspace_bytes()";
         case FP8BS_ERR_TOO_LARGE: return "operand exceeds the 4 GiB buffer-addressing limit (m*k or n*k >= 2^32)";
         case FP8BS_ERR_LAUNCH: return "kernel launch failed";
@@ -170,6 +178,10 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
     hipStream_t s = (hipStream_t)stream;
     fp8bs_plan_t plan{};
     if (k == 0) variant = FP8BS_VARIANT_GENERIC;   // empty sum: the generic kernel writes zeros
+    if (!vector_aligned(a, b, c, ws)) {
+        if (variant != FP8BS_VARIANT_AUTO && variant != FP8BS_VARIANT_GENERIC) return FP8BS_ERR_BAD_VARIANT;
+        variant = FP8BS_VARIANT_GENERIC;
+    }
     if (variant == FP8BS_VARIANT_AUTO) {
         choose(m, n, k, 0, &plan);
         if (split_k > 0) fill_plan(m, n, k, plan.variant, split_k, &plan);
@@ -216,7 +228,7 @@ int fp8bs_gemm_grouped(const void* a, const void* b, const float* a_scale, const
     g.c = (uint16_t*)c; g.ws = nullptr; g.row_offsets = row_offsets;
     g.m = total_rows; g.n = n; g.k = k; g.lda = total_rows; g.nb = (n + 127) / 128;
     g.split_k = 1; g.kb_per_split = k / KBLK; g.band_h = 4; g.num_experts = num_experts;
-    int variant = (k == 0 || (total_rows % 16) != 0 || (n % 16) != 0) ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
+    int variant = (k == 0 || (total_rows % 16) != 0 || (n % 16) != 0 || !vector_aligned(a, b, c, nullptr)) ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
     if (fp8bs::launch_gemm(variant, 2, g, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
     return FP8BS_OK;
 }
@@ -235,7 +247,7 @@ int fp8bs_gemm_silu_mul(const void* a, const void* b, const float* a_scale, cons
     g.split_k = 1; g.kb_per_split = k / KBLK; g.band_h = 4; g.num_experts = row_offsets ? num_experts : 0;
     g.epi = 1;
     // 16-byte stores of n/2-wide bf16 rows need n % 16 == 0 as the copies do
-    int variant = (k == 0 || (rows % 16) != 0 || (n % 16) != 0) ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
+    int variant = (k == 0 || (rows % 16) != 0 || (n % 16) != 0 || !vector_aligned(a, b, h, nullptr)) ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
     if (fp8bs::launch_gemm(variant, row_offsets ? 2 : 0, g, (hipStream_t)stream) != hipSuccess) return FP8BS_ERR_LAUNCH;
     return FP8BS_OK;
 }

@@ -32,7 +32,8 @@ extern "C" {
 enum {
     FP8BS_OK = 0,
     FP8BS_ERR_NULL_POINTER = 1,   /* a required pointer is NULL                             */
-    FP8BS_ERR_BAD_SHAPE = 2,      /* m,n,k <= 0 where not allowed, or k % 128 != 0           */
+    FP8BS_ERR_BAD_SHAPE = 2,      /* m,n,k <= 0 where not allowed, k % 128 != 0, or a pointer
+                                     not aligned to its element type                          */
     FP8BS_ERR_WORKSPACE = 3,      /* ws is NULL / smaller than fp8bs_workspace_bytes(...)    */
     FP8BS_ERR_TOO_LARGE = 4,      /* an operand exceeds the 4 GiB buffer-addressing limit    */
     FP8BS_ERR_LAUNCH = 5,         /* hipGetLastError() after launch was not hipSuccess       */
@@ -84,7 +85,10 @@ size_t fp8bs_workspace_bytes(int m, int n, int k);
 
 /* Dense GEMM. Replaces `fp8_mm(a,b,as,bs,c,c_tmp)`,
  * 1-amd-fp8-mm/amd-fp8-mm-submission.py:514-579. Inputs are never modified (the reference's
- * pre-transpose branch, :570-571, overwrites a and b; this one does not). */
+ * pre-transpose branch, :570-571, overwrites a and b; this one does not).
+ * Alignment: the fast kernels need m and n multiples of 16 and a, b, c, ws on 16-byte boundaries;
+ * other shapes or pointers run on the element-wise generic kernel (correct, slow).  a_scale and
+ * b_scale must be 4-byte aligned, c 2-byte aligned (FP8BS_ERR_BAD_SHAPE otherwise). */
 int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
                void* c, void* ws, size_t ws_bytes, int m, int n, int k, void* stream);
 

@@ -87,6 +87,33 @@ def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
             _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d" % (m, n, k, variant))
 
 
+def _shifted(t, nbytes):
+    """A copy of K-major / contiguous ``t`` whose storage starts ``nbytes`` past a 256-byte boundary."""
+    rows_major = t.t() if t.stride(0) == 1 and t.dim() == 2 and t.shape[0] > 1 else t
+    flat = torch.empty(rows_major.numel() * t.element_size() + 256, dtype=torch.uint8, device=t.device)
+    view = flat[nbytes:nbytes + rows_major.numel() * t.element_size()].view(t.dtype).view(rows_major.shape)
+    view.copy_(rows_major)
+    return view.t() if rows_major is not t else view
+
+
+@pytest.mark.parametrize("which", ["a", "b", "c"])
+def test_pointers_off_the_16_byte_grid_take_the_generic_kernel(pkg, oracle, dev, which):
+    """The vector kernels need 16-byte aligned operands; anything else must still give the right answer."""
+    cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0], m=64, n=128, k=256)
+    a, b, a_scale, b_scale, c = _to(cpu, dev)
+    if which == "a":
+        a = _shifted(a, 4)
+    elif which == "b":
+        b = _shifted(b, 8)
+    else:
+        c = _shifted(c, 2)
+    assert (a.data_ptr() | b.data_ptr() | c.data_ptr()) % 16 != 0
+    out = pkg.custom_kernel((a, b, a_scale, b_scale, c))
+    _check(oracle, out, oracle.ref_kernel(cpu), "misaligned " + which)
+    with pytest.raises(RuntimeError):
+        pkg.custom_kernel((a, b, a_scale, b_scale, c), variant=2, split_k=1)     # a forced vector kernel is refused
+
+
 def test_empty_shapes(pkg, dev):
     cfg = pkg.inputs.CONFIGS[0]
     a, b, a_scale, b_scale, c = _to(pkg.inputs.make_dense(cfg, m=32, n=64, k=128), dev)
