@@ -308,6 +308,7 @@ extern "C" int fp8bs_moe_combine(const void* y, int rows, const int32_t* slot_of
     if (tokens < 0 || rows < 0 || topk <= 0 || d < 0 || (d % 8) != 0) return FP8BS_ERR_BAD_SHAPE;
     if (tokens == 0 || d == 0) return FP8BS_OK;
     if (!y || !slot_of || !weights || !out) return FP8BS_ERR_NULL_POINTER;
+    if ((((uintptr_t)y | (uintptr_t)out) & 15) != 0) return FP8BS_ERR_BAD_SHAPE;      // 16-byte row accesses
     hipLaunchKernelGGL(fp8bs::moe_combine_kernel, dim3(tokens), dim3(fp8bs::RB), 0, (hipStream_t)stream,
                        (const uint16_t*)y, slot_of, weights, (uint16_t*)out, rows, topk, d);
     return hipGetLastError() == hipSuccess ? FP8BS_OK : FP8BS_ERR_LAUNCH;

@@ -185,7 +185,7 @@ int fp8bs_gemm_silu_mul(const void* a, const void* b, const float* a_scale, cons
                         const int32_t* row_offsets, int num_experts, int rows, int n, int k, void* stream);
 
 /* Weighted un-permute: out[t][:] = sum_j weights[t][j] * y[slot_of[t][j]][:]  (y bf16 [rows][d], out bf16
- * [tokens][d], d % 8 == 0; fp32 accumulation in the order j = 0..topk-1, one rounding; a slot outside
+ * [tokens][d], d % 8 == 0, y and out 16-byte aligned; fp32 accumulation in the order j = 0..topk-1, one rounding; a slot outside
  * [0, rows) is skipped).  Role of pack_output (2-amd-moe/amd-moe-submission.py:239-301; fp16
  * accumulation there). */
 int fp8bs_moe_combine(const void* y, int rows, const int32_t* slot_of, const float* weights, void* out,
