@@ -57,12 +57,16 @@ void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out)
     out->workspace_bytes = split_k > 1 ? (uint64_t)split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
 }
 
-// Shape-family rule.  m or n not a multiple of 16 -> generic kernel (the tiled kernels copy 16-byte
-// chunks along m and n).  m > 128 -> the tiled MFMA kernel whose tile shape finishes soonest under a
+// What the vector kernels need of a shape: rows of a (m bytes) that keep the 4-byte loads of a copy
+// aligned and inside the buffer's per-dword range check, rows of c (n bf16) that keep 16-byte stores
+// aligned.
+bool vector_shape(int m, int n) { return (m % 4) == 0 && (n % 8) == 0; }
+
+// Shape-family rule.  m not a multiple of 4 or n not a multiple of 8 -> generic kernel.  m > 128 -> the tiled MFMA kernel whose tile shape finishes soonest under a
 // small cost model.  m <= 128 -> the streaming kernel with the K split that fills the CUs.
 void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     if (num_cus <= 0) num_cus = 256;
-    if ((m % 16) != 0 || (n % 16) != 0) { fill_plan(m, n, k, FP8BS_VARIANT_GENERIC, 1, out); return; }
+    if (!vector_shape(m, n)) { fill_plan(m, n, k, FP8BS_VARIANT_GENERIC, 1, out); return; }
     int kbt = k / KBLK;
     if (m > 128) {
         // Compute-bound family: the tile shape and K split that finish soonest under a cost model in
@@ -188,7 +192,7 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
     } else {
         VariantInfo vi{};
         if (!variant_info(variant, &vi)) return FP8BS_ERR_BAD_VARIANT;
-        if (variant != FP8BS_VARIANT_GENERIC && ((m % 16) != 0 || (n % 16) != 0)) return FP8BS_ERR_BAD_VARIANT;
+        if (variant != FP8BS_VARIANT_GENERIC && !vector_shape(m, n)) return FP8BS_ERR_BAD_VARIANT;
         fill_plan(m, n, k, variant, split_k > 0 ? split_k : 1, &plan);
     }
     if (plan.split_k > 1 && (!ws || ws_bytes < plan.workspace_bytes)) return FP8BS_ERR_WORKSPACE;
@@ -228,7 +232,7 @@ int fp8bs_gemm_grouped(const void* a, const void* b, const float* a_scale, const
     g.c = (uint16_t*)c; g.ws = nullptr; g.row_offsets = row_offsets;
     g.m = total_rows; g.n = n; g.k = k; g.lda = total_rows; g.nb = (n + 127) / 128;
     g.split_k = 1; g.kb_per_split = k / KBLK; g.band_h = 4; g.num_experts = num_experts;
-    int variant = (k == 0 || (total_rows % 16) != 0 || (n % 16) != 0 || !vector_aligned(a, b, c, nullptr)) ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
+    int variant = (k == 0 || !vector_shape(total_rows, n) || !vector_aligned(a, b, c, nullptr)) ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
     if (fp8bs::launch_gemm(variant, 2, g, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
     return FP8BS_OK;
 }
@@ -246,8 +250,8 @@ int fp8bs_gemm_silu_mul(const void* a, const void* b, const float* a_scale, cons
     g.m = rows; g.n = n; g.k = k; g.lda = rows; g.nb = (n + 127) / 128;
     g.split_k = 1; g.kb_per_split = k / KBLK; g.band_h = 4; g.num_experts = row_offsets ? num_experts : 0;
     g.epi = 1;
-    // 16-byte stores of n/2-wide bf16 rows need n % 16 == 0 as the copies do
-    int variant = (k == 0 || (rows % 16) != 0 || (n % 16) != 0 || !vector_aligned(a, b, h, nullptr)) ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
+    // 16-byte stores of n/2-wide bf16 rows need n % 16 == 0
+    int variant = (k == 0 || !vector_shape(rows, n) || (n % 16) != 0 || !vector_aligned(a, b, h, nullptr)) ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
     if (fp8bs::launch_gemm(variant, row_offsets ? 2 : 0, g, (hipStream_t)stream) != hipSuccess) return FP8BS_ERR_LAUNCH;
     return FP8BS_OK;
 }

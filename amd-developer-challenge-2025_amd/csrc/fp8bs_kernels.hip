@@ -241,8 +241,10 @@ void gemm_tr_kernel(const GemmArgs p) {
     // slot P = that + l, which holds k row P/CPR, stored chunk P%CPR = logical chunk (P%CPR) ^ swz(k row).
     // The XOR mask of a lane does not depend on q, so a lane's global offset is one constant (k row of
     // copy 0, chunk column) plus a wave-uniform term (k block and q), which travels in an SGPR.
-    // Chunk columns beyond the matrix are clamped to its last 16 rows: such rows are never stored,
-    // and every address the copies form stays inside the operand.
+    // A chunk that starts beyond the matrix is pointed at the tile's first chunk (its rows are never
+    // stored).  A chunk that starts inside and ends beyond it (m a multiple of 4 but not of 16) runs on
+    // into the next k row, or, in the last k row, past the end of the buffer, where the per-dword range
+    // check of the buffer load returns zeros: the rows that exist are always read from where they are.
     // a_scale row of a k block: BM floats, copied 64 floats (one dword per lane) per wave into the tail
     // of the stage.  Every wave issues the copy (wave w the same 64 floats as wave w % (BM/64), to the
     // same place): a branch here would split the K loop's straight-line block and the compiler would
@@ -260,11 +262,11 @@ void gemm_tr_kernel(const GemmArgs p) {
         int P = wave * 64 + lane;
         int krow = P / C::CPR_A, ch = (P % C::CPR_A) ^ swz_of_krow<C::CPR_A>(krow);
         int col = t.m0 + 16 * ch;
-        col = col < p.lda - 16 ? col : p.lda - 16;
+        col = col < p.lda ? col : t.m0;
         c.a_voff = (uint32_t)krow * (uint32_t)p.lda + (uint32_t)col;
         krow = P / C::CPR_B; ch = (P % C::CPR_B) ^ swz_of_krow<C::CPR_B>(krow);
         col = t.n0 + 16 * ch;
-        col = col < p.n - 16 ? col : p.n - 16;
+        col = col < p.n ? col : t.n0;
         c.b_voff = (uint32_t)krow * (uint32_t)p.n + (uint32_t)col;
         int r = t.m0 + as_wave * 64 + lane;
         r = r < p.lda - 1 ? r : p.lda - 1;
@@ -617,8 +619,8 @@ void gemm_skinny_kernel(const GemmArgs p) {
     // ---- copy plan.  The one-KiB copies of a block are numbered I = 4q + wave, q = 0..COPIES-1:
     //      I < A_COPIES the A tile, then B_COPIES of the B tile (copy Ib fills B chunks 64*Ib ..), then the
     //      a_scale row, then the b_scale values (repeated as padding).  Lane offsets are fixed for the
-    //      whole kernel; the K block enters through the wave-uniform offset.  Columns beyond the matrix
-    //      are clamped (never stored).
+    //      whole kernel; the K block enters through the wave-uniform offset.  Chunks that start beyond
+    //      the matrix re-read the tile's first chunk (never stored).
     uint32_t voff[C::COPIES];
 #pragma unroll
     for (int q = 0; q < C::COPIES; q++) {
@@ -628,14 +630,14 @@ void gemm_skinny_kernel(const GemmArgs p) {
             int krow = 16 * I + lane / 4;
             int c = (lane % 4) ^ swz_of_krow<C::CPR_A>(krow);
             int col = m0 + 16 * c;
-            col = col < p.lda - 16 ? col : p.lda - 16;
+            col = col < p.lda ? col : m0;
             v = (uint32_t)krow * (uint32_t)p.lda + (uint32_t)col;
         } else if (I < C::A_COPIES + C::B_COPIES) {
             int P = 64 * (I - C::A_COPIES) + lane;
             int kr = P / C::CPR_B, cc = P % C::CPR_B;
             if (C::SWZ_B) cc ^= swz_of_krow<C::CPR_B>(kr);
             int cl = n0 + 16 * cc;
-            cl = cl < p.n - 16 ? cl : p.n - 16;
+            cl = cl < p.n ? cl : n0;
             v = (uint32_t)kr * (uint32_t)p.n + (uint32_t)cl;
         } else if (I == C::A_COPIES + C::B_COPIES) {
             int r = m0 + lane; r = r < p.lda - 1 ? r : p.lda - 1;
