@@ -25,6 +25,23 @@ struct GemmArgs {
     int epi;                // 0: bf16 of the product; 1: silu(column 2i) * column 2i+1, n/2 output columns
 };
 
+// Per-device bookkeeping of the launchers.  A kernel's dynamic-LDS limit is a property of the kernel
+// on one device, so "already raised" is remembered per device; devices beyond the table just set the
+// attribute on every launch.  Races between threads are harmless (the call is idempotent).
+static constexpr int MAX_DEVICES = 64;
+inline int device_slot() {
+    int d = 0;
+    return (hipGetDevice(&d) == hipSuccess && d >= 0 && d < MAX_DEVICES) ? d : -1;
+}
+// `raised[slot]` holds the largest limit set so far for this kernel on that device.
+inline hipError_t raise_lds_limit(const void* kernel, int bytes, int* raised) {
+    const int slot = device_slot();
+    if (slot >= 0 && raised[slot] >= bytes) return hipSuccess;
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess && slot >= 0) raised[slot] = bytes;
+    return e;
+}
+
 // mode: 0 dense bf16, 1 dense split-K partials, 2 grouped.  variant: FP8BS_VARIANT_* (not AUTO).
 hipError_t launch_gemm(int variant, int mode, const GemmArgs& args, hipStream_t stream);
 hipError_t launch_splitk_reduce(const float* ws, uint16_t* c, size_t mn, int split_k, hipStream_t stream);

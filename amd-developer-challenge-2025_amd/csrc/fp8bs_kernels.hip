@@ -834,25 +834,22 @@ template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0>
 static hipError_t launch_tr(const GemmArgs& a, dim3 grid, hipStream_t stream) {
     using C = TileCfg<BM, BN, WM, WN, MODE>;
     auto kern = gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI>;
-    static bool attr_done = false;   // raising the dynamic-LDS limit is idempotent; a race is harmless
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    static int raised[MAX_DEVICES];
+    hipError_t e = raise_lds_limit((const void*)kern, C::LDS_BYTES, raised);
+    if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, grid, dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
     return hipGetLastError();
 }
 
-// CUs of the current device (asked once per process and device change is not expected mid-run)
+// CUs of the current device (asked once per device)
 static int device_cus() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
-        else cus = 256;
-    }
-    return cus;
+    static int cus[MAX_DEVICES];
+    const int slot = device_slot();
+    if (slot >= 0 && cus[slot] > 0) return cus[slot];
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    if (slot >= 0) cus[slot] = n;
+    return n;
 }
 
 template <int BM, int BN, int WM, int WN, bool WITH_EPI = false>
@@ -893,13 +890,9 @@ static hipError_t launch_skinny(const GemmArgs& a, int mode, hipStream_t stream)
     using C = SkinnyCfg<BN, NSTAGE>;
     auto k0 = gemm_skinny_kernel<BN, NSTAGE, 0>;
     auto k1 = gemm_skinny_kernel<BN, NSTAGE, 1>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void*)k0, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    static int raised0[MAX_DEVICES], raised1[MAX_DEVICES];
+    hipError_t e = mode == 1 ? raise_lds_limit((const void*)k1, C::LDS_BYTES, raised1) : raise_lds_limit((const void*)k0, C::LDS_BYTES, raised0);
+    if (e != hipSuccess) return e;
     int tiles = ((a.n + C::BN - 1) / C::BN) * a.split_k * ((a.m + C::BM - 1) / C::BM);
     if (mode == 1) hipLaunchKernelGGL(k1, dim3(tiles), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
     else hipLaunchKernelGGL(k0, dim3(tiles), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);

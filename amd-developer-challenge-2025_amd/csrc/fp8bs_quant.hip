@@ -24,6 +24,7 @@
 #include <stddef.h>
 
 #include "fp8bs.h"
+#include "fp8bs_kernels.h"
 
 namespace fp8bs {
 
@@ -385,11 +386,10 @@ static hipError_t launch_gather(const GatherArgs& a, hipStream_t stream) {
     const int quarter = (a.src_rows + 3) / 4;
     const int lds = 4 * quarter * KC;
     auto kern = gather_a_kernel<KC>;
-    static int attr_lds = 0;     // largest dynamic-LDS size allowed so far; raising it again is harmless
-    if (lds > 65536 && lds > attr_lds) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    static int raised[MAX_DEVICES];
+    if (lds > 65536) {
+        hipError_t e = raise_lds_limit((const void*)kern, lds, raised);
         if (e != hipSuccess) return e;
-        attr_lds = lds;
     }
     dim3 grid((unsigned)(a.k / KC), (unsigned)((a.rows + a.rows_per_wg - 1) / a.rows_per_wg));
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
