@@ -134,8 +134,8 @@ int check_common(const void* a, const void* b, const float* as, const float* bs,
 }
 
 // The tiled and streaming kernels copy and store 16 bytes at a time: operands, output and workspace
-// must start on 16-byte boundaries (rows then do too, because m and n are multiples of 16 there).
-// Anything else is left to the generic kernel, which accesses single elements.
+// must start on 16-byte boundaries (with vector_shape() the copies then stay dword-aligned and the
+// stores 16-byte aligned).  Anything else is left to the generic kernel, which accesses single elements.
 bool vector_aligned(const void* a, const void* b, const void* c, const void* ws) {
     return ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)ws) & 15) == 0);
 }

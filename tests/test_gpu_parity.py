@@ -3,6 +3,7 @@
 Bar: every output element within |out - ref| <= 1e-3 + 2e-2*|ref| of the oracle
 (dequantise -> fp32 matmul -> bf16).  Run with:  python -u -m pytest tests -m gpu
 """
+import numpy as np
 import pytest
 import torch
 
@@ -88,6 +89,31 @@ def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
         for variant in (2, 3, 4, 5, 6, 7, 8):
             out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1)
             _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d" % (m, n, k, variant))
+
+
+def test_seeded_random_shapes_through_the_planner(pkg, oracle, dev):
+    """40 seeded shapes on the 4 x 8 grid of the vector kernels, whatever the planner picks for each
+    (tile shape, K split, streaming kernel), plus one forced K split per shape."""
+    rng = np.random.default_rng(20259)
+    cfg = pkg.inputs.CONFIGS[2]                                   # outlier activations, small weights
+    seen = set()
+    for i in range(40):
+        if i % 4 == 3:                                            # large enough for the big tiles
+            m, n = 4 * int(rng.integers(256, 1200)), 8 * int(rng.integers(128, 500))
+        else:
+            m = int(rng.choice([4, 8, 12, 16])) * int(rng.integers(1, 60)) if i % 3 else 4 * int(rng.integers(1, 40))
+            n = 8 * int(rng.integers(1, 140))
+        k = 128 * int(rng.integers(1, 13))
+        cpu = pkg.inputs.make_dense(cfg, m=m, n=n, k=k)
+        ref = oracle.ref_kernel(cpu)
+        plan = pkg.plan(m, n, k)
+        seen.add((plan.variant, plan.split_k > 1))
+        out = pkg.custom_kernel(_to(cpu, dev))
+        _check(oracle, out, ref, "shape %dx%dx%d planned variant %d split %d" % (m, n, k, plan.variant, plan.split_k))
+        split = int(rng.integers(2, 6))
+        out = pkg.custom_kernel(_to(cpu, dev), variant=plan.variant, split_k=split)
+        _check(oracle, out, ref, "shape %dx%dx%d variant %d forced split %d" % (m, n, k, plan.variant, split))
+    assert len({v for v, _ in seen}) >= 4, "the draw should reach several kernel variants: %s" % sorted(seen)
 
 
 def _shifted(t, nbytes):
