@@ -35,6 +35,7 @@ namespace fp8bs {
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
@@ -112,7 +113,9 @@ struct TileCfg {
     static constexpr int CPR_A = BM / 16, CPR_B = BN / 16;          // 16-byte chunks per k row
     static constexpr int A_BYTES = KBLK * BM, B_BYTES = KBLK * BN;
     static constexpr int AS_BYTES = BM * 4;                          // the k block's a_scale row
-    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + (AS_BYTES < 1024 ? 1024 : AS_BYTES);
+    static constexpr int AS_AREA = AS_BYTES < 1024 ? 1024 : AS_BYTES;
+    static constexpr int BS_AREA = 256;                              // the k block's b_scale values of the tile's n blocks
+    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + AS_AREA + BS_AREA;
     static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
     static constexpr int A_LOADS = A_BYTES / 16 / NTHREADS;         // 16-byte loads per thread per block
     static constexpr int B_LOADS = B_BYTES / 16 / NTHREADS;
@@ -120,6 +123,11 @@ struct TileCfg {
     static_assert(WN <= 128 && 128 % WN == 0, "a wave's n range must stay inside one b_scale block");
     static_assert(CPR_A <= 16 && CPR_B <= 16, "swizzle assumes a k row spans at most 256 bytes");
 };
+
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    // s_waitcnt with only vmcnt constrained: vmcnt is split over bits [3:0] and [15:14]
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
 
 template <int CPR>
 __device__ __forceinline__ int swz_of_krow(int krow) {
@@ -142,6 +150,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64)
 void gemm_tr_kernel(const GemmArgs p) {
     using C = TileCfg<BM, BN, WM, WN, MODE>;
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+
+    // global store instructions per wave and tile in the bf16 epilogue (always this many: lanes without
+    // a valid element are switched off by an out-of-range buffer offset, not by a branch)
+    constexpr int EPI_WNO = EPI == 1 ? WN / 2 : WN;
+    constexpr int EPI_STORES = MODE == 1 ? 0 : 2 * ((WM / 2) * (EPI_WNO * 2 / 16) / 64);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -234,7 +247,6 @@ void gemm_tr_kernel(const GemmArgs p) {
     const uint32_t a_bytes = (uint32_t)p.k * (uint32_t)p.lda;
     const uint32_t b_bytes = (uint32_t)p.k * (uint32_t)p.n;
     __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, a_bytes, 0x00020000);
-    __amdgpu_buffer_rsrc_t as_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.as, 0, (uint32_t)(p.k / KBLK) * (uint32_t)p.lda * 4u, 0x00020000);
 
     // ---- global -> LDS copy plan of a tile -------------------------------------------------------
     // Wave w, copy q fills the 1 KiB of LDS that starts at chunk slot (q*NWAVES + w)*64; lane l fills
@@ -245,17 +257,23 @@ void gemm_tr_kernel(const GemmArgs p) {
     // stored).  A chunk that starts inside and ends beyond it (m a multiple of 4 but not of 16) runs on
     // into the next k row, or, in the last k row, past the end of the buffer, where the per-dword range
     // check of the buffer load returns zeros: the rows that exist are always read from where they are.
-    // a_scale row of a k block: BM floats, copied 64 floats (one dword per lane) per wave into the tail
-    // of the stage.  Every wave issues the copy (wave w the same 64 floats as wave w % (BM/64), to the
-    // same place): a branch here would split the K loop's straight-line block and the compiler would
-    // sink the folds of the first MFMAs below it, away from the MFMAs they are meant to overlap.
+    // Scales of a k block ride along in the tail of the stage: the a_scale row (BM floats, 64 per wave,
+    // waves 0 .. BM/64-1) and the b_scale values of the tile's n blocks (the remaining waves, all the same
+    // copy to the same place).  Every wave issues exactly one such 4-byte-per-lane copy, with its source
+    // and destination in scalar registers: a branch here would split the K loop's straight-line block and
+    // the compiler would sink the folds of the first MFMAs below it, away from the MFMAs they are meant
+    // to overlap.  With the scales in LDS the K loop has no loads of its own that the compiler would have
+    // to order against the output stores of the previous tile.
     constexpr int ROWS_PER_COPY_A = C::NWAVES * 64 / C::CPR_A, ROWS_PER_COPY_B = C::NWAVES * 64 / C::CPR_B;
     constexpr int AS_COPIES = BM / 64;
-    const int as_wave = wave % AS_COPIES;
+    static_assert(C::NWAVES > AS_COPIES, "some wave must be left to copy the b_scale values");
+    const bool sc_is_b = wave >= AS_COPIES;                       // this wave's scale copy is the b_scale one
+    const uint32_t sc_dst = C::A_BYTES + C::B_BYTES + (sc_is_b ? C::AS_AREA : wave * 256);
+    const uint32_t sc_kstep = (sc_is_b ? (uint32_t)p.nb : (uint32_t)p.lda) * 4u;
     struct CopyPlan {
-        uint32_t a_voff, b_voff, as_voff;
+        uint32_t a_voff, b_voff, sc_voff;
         int kb_begin;
-        __amdgpu_buffer_rsrc_t b_rsrc;
+        __amdgpu_buffer_rsrc_t b_rsrc, sc_rsrc;
     };
     auto copy_plan = [&](const Tile& t) -> CopyPlan {
         CopyPlan c;
@@ -268,11 +286,14 @@ void gemm_tr_kernel(const GemmArgs p) {
         col = t.n0 + 16 * ch;
         col = col < p.n ? col : t.n0;
         c.b_voff = (uint32_t)krow * (uint32_t)p.n + (uint32_t)col;
-        int r = t.m0 + as_wave * 64 + lane;
-        r = r < p.lda - 1 ? r : p.lda - 1;
-        c.as_voff = (uint32_t)r * 4u;
+        int r = sc_is_b ? t.n0 / 128 + lane : t.m0 + wave * 64 + lane;      // n block or row of a
+        const int last = (sc_is_b ? p.nb : p.lda) - 1;
+        r = r < last ? r : last;
+        c.sc_voff = (uint32_t)r * 4u;
         c.kb_begin = t.kb_begin;
         c.b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.bptr, 0, b_bytes, 0x00020000);
+        c.sc_rsrc = __builtin_amdgcn_make_buffer_rsrc(sc_is_b ? (void*)t.bsptr : (void*)p.as, 0,
+                                                      (uint32_t)(p.k / KBLK) * (sc_is_b ? (uint32_t)p.nb : (uint32_t)p.lda) * 4u, 0x00020000);
         return c;
     };
     const uint32_t a_kstep = (uint32_t)KBLK * (uint32_t)p.lda, b_kstep = (uint32_t)KBLK * (uint32_t)p.n;
@@ -282,7 +303,7 @@ void gemm_tr_kernel(const GemmArgs p) {
     // stage and would otherwise make every LDS read wait for all outstanding copies.  Completion is
     // enforced by hand: s_waitcnt vmcnt(0) + workgroup barrier before the first read of a stage.
     const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
-    constexpr int NLOADS = C::A_LOADS + C::B_LOADS + 1;     // + the a_scale row
+    constexpr int NLOADS = C::A_LOADS + C::B_LOADS + 1;     // + the scales
     // copy q (compile-time) of k block `blk` (relative to the tile's first) into `stage`
     auto issue_one = [&](const CopyPlan& cp, int stage, int blk, auto q_tag) {
         constexpr int q = decltype(q_tag)::value;
@@ -294,7 +315,7 @@ void gemm_tr_kernel(const GemmArgs p) {
             constexpr int qb = q - C::A_LOADS;
             copy16_global_to_lds(cp.b_rsrc, sa + C::A_BYTES + qb * C::NWAVES * 1024, cp.b_voff, kb * b_kstep + (uint32_t)(qb * ROWS_PER_COPY_B) * (uint32_t)p.n);
         } else {
-            copy4_global_to_lds(as_rsrc, lds_base + stage * C::STAGE_BYTES + C::A_BYTES + C::B_BYTES + as_wave * 256, cp.as_voff, kb * (uint32_t)p.lda * 4u);
+            copy4_global_to_lds(cp.sc_rsrc, lds_base + stage * C::STAGE_BYTES + sc_dst, cp.sc_voff, kb * sc_kstep);
         }
     };
     auto issue_all = [&](const CopyPlan& cp, int stage, int blk) {
@@ -330,21 +351,18 @@ void gemm_tr_kernel(const GemmArgs p) {
     };
 
     const int as_lane_off = C::A_BYTES + C::B_BYTES + (wave_m * WM + i16) * 4;
+    const int bs_off = C::A_BYTES + C::B_BYTES + C::AS_AREA + (wave_n * WN / 128) * 4;   // a wave's n range lies inside one 128-block
 
     Tile cur = pick_tile(0);
     if (!cur.valid) return;
     CopyPlan cp = copy_plan(cur);
     bool prefetched = false;                // block 0 of `cur` is already on its way into stage 0
+    bool stores_behind = false;             // ... and this wave's output stores of the previous tile were issued after it
     for (int it = 0;; it++) {
     const int m0 = cur.m0, n0 = cur.n0, kb_begin = cur.kb_begin, kb_end = cur.kb_end, split_z = cur.split_z;
     const int row_lo = cur.row_lo, row_hi = cur.row_hi;
-    const float* bsptr = cur.bsptr;
-    // ---- scales -------------------------------------------------------------------------------
     // a_scale: lane's output row of m-tile t is tile row wave_m*WM + 16t + i16, read from the stage's
-    // copy of the a_scale row.  b_scale: one value per wave and k block (a wave's n range lies inside
-    // one 128-block), loaded straight from memory two k blocks ahead.
-    int nblk = (n0 + wave_n * WN) / 128;
-    nblk = __builtin_amdgcn_readfirstlane(nblk < p.nb - 1 ? nblk : p.nb - 1);
+    // copy of the a_scale row.
     // does any row of this wave's tile get stored?
     const bool wave_active = __builtin_amdgcn_readfirstlane((m0 + wave_m * WM < row_hi && m0 + wave_m * WM + WM > row_lo) ? 1 : 0) != 0;
 
@@ -369,11 +387,12 @@ void gemm_tr_kernel(const GemmArgs p) {
         // ---- prologue: block 0 -> stage 0 (unless the previous tile already sent it), wait; first
         //      copies of block 1 -> stage 1.  The barrier also ends the previous tile's use of stage 1
         //      as the staging area of its output ----
-        const float* bs_ptr = bsptr + (size_t)kb_begin * p.nb + nblk;   // b_scale of the current k block
-        float bs_cur = bs_ptr[0];
-        float bs_nxt = nkb > 1 ? bs_ptr[p.nb] : 0.f;
+        // The vector memory counter retires loads and stores in the order they were issued.  If block 0
+        // was sent ahead of the previous tile's NSTORES output stores, "at most NSTORES outstanding" means
+        // the block has landed, and the stores are left to finish under the first K block.
         if (!prefetched) issue_all(cp, 0, 0);
-        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+        if (prefetched && stores_behind) wait_vmcnt<EPI_STORES>();
+        else wait_vmcnt<0>();
         __syncthreads();
         if (nkb > 1) {
             [&]<int... Q>(std::integer_sequence<int, Q...>) {
@@ -414,10 +433,9 @@ void gemm_tr_kernel(const GemmArgs p) {
             const unsigned char* sbase = lds + cur_stage * C::STAGE_BYTES;
             const unsigned char* snext = lds + (cur_stage ^ 1) * C::STAGE_BYTES;
             float sc[C::MT];
+            const float bsv = *(const float*)(sbase + bs_off);
 #pragma unroll
-            for (int t = 0; t < C::MT; t++) sc[t] = *(const float*)(sbase + as_lane_off + t * 64) * bs_cur;
-            bs_cur = bs_nxt;
-            if constexpr (HAS_NEXT2) bs_nxt = bs_ptr[(size_t)(j + 2) * p.nb];
+            for (int t = 0; t < C::MT; t++) sc[t] = *(const float*)(sbase + as_lane_off + t * 64) * bsv;
             v4f ring[RING];
             auto step = [&](auto s_tag) {
                 constexpr int s = decltype(s_tag)::value;
@@ -504,6 +522,15 @@ void gemm_tr_kernel(const GemmArgs p) {
         static_assert(C::MT % 2 == 0 && C::NWAVES * HALF_ROWS * WNO * 2 <= C::STAGE_BYTES, "output staging must fit one stage");
         unsigned char* region = lds + C::STAGE_BYTES + wave * (HALF_ROWS * WNO * 2);
         const int ldc = EPI == 1 ? p.n / 2 : p.n;
+        // Stores go through buffer descriptors: an offset of 0xFFFFFFFF drops the lane's store, so the
+        // instruction count does not depend on the data.  Each store gets a descriptor based at the first
+        // element of its group of rows (scalar arithmetic only); the scalar-offset operand is not used:
+        // with it, the vector ALU instruction that follows a 16-byte store was seen to overwrite the
+        // store's data register before the store had read it (the compiler pads that case only for
+        // stores without a scalar offset).
+        const int col0 = EPI == 1 ? n0 / 2 : n0;
+        uint16_t* const c_tile = p.c + (size_t)m0 * ldc + col0;
+        static_assert(MODE == 1 || EPI_STORES == 2 * (HALF_ROWS * ROW_CHUNKS / 64), "store count used by the next tile's wait");
 #pragma unroll
         for (int half = 0; half < 2; half++) {
 #pragma unroll
@@ -526,22 +553,29 @@ void gemm_tr_kernel(const GemmArgs p) {
                     }
                 }
             }
-            constexpr int PASSES = HALF_ROWS * ROW_CHUNKS / 64;
-            static_assert(HALF_ROWS * ROW_CHUNKS % 64 == 0, "a half tile is a whole number of 16-byte sweeps");
+            constexpr int PASSES = HALF_ROWS * ROW_CHUNKS / 64, ROWS_PER_PASS = 64 / ROW_CHUNKS;
+            static_assert(HALF_ROWS * ROW_CHUNKS % 64 == 0 && 64 % ROW_CHUNKS == 0, "a half tile is a whole number of 16-byte sweeps");
+            // lane -> (row inside the pass, chunk); everything else about a store's address is uniform
+            // and sits in the descriptor, so the 16 stores need one address register, not 16
+            const int lane_r = lane / ROW_CHUNKS, lane_chunk = lane % ROW_CHUNKS;
+            const int wave_row0 = wave_m * WM, wave_col0 = wave_n * WNO;              // inside the tile, output columns
+            const bool col_ok = col0 + wave_col0 + lane_chunk * 8 < ldc;
+            const uint32_t lane_off = ((uint32_t)(wave_row0 + lane_r) * (uint32_t)ldc + (uint32_t)(wave_col0 + lane_chunk * 8)) * 2u;
 #pragma unroll
             for (int q = 0; q < PASSES; q++) {
-                const int idx = q * 64 + lane;
-                const int r = idx / ROW_CHUNKS, chunk = idx % ROW_CHUNKS;
+                const int r = q * ROWS_PER_PASS + lane_r;
                 const int sw = (r / ROWS_PER_SWEEP) % ROW_CHUNKS;
-                const v4i val = *(const v4i*)(region + r * (WNO * 2) + ((chunk ^ sw) << 4));
-                const int row = m0 + wave_m * WM + half * HALF_ROWS + r;
-                const int col = (EPI == 1 ? (n0 + wave_n * WN) / 2 : n0 + wave_n * WN) + chunk * 8;
-                if (row >= row_lo && row < row_hi && col < ldc)
-                    __builtin_nontemporal_store(val, (v4i*)(p.c + (size_t)row * ldc + col));   // written once, not read again here
+                const v4i val = *(const v4i*)(region + r * (WNO * 2) + ((lane_chunk ^ sw) << 4));
+                const int pass_row0 = half * HALF_ROWS + q * ROWS_PER_PASS;            // compile-time
+                const int row = m0 + wave_row0 + pass_row0 + lane_r;
+                const bool ok = col_ok && row >= row_lo && row < row_hi;
+                __amdgpu_buffer_rsrc_t c_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(c_tile + (size_t)pass_row0 * ldc), 0, 0xFFFFFFF0u, 0x00020000);
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, val), c_rsrc, ok ? lane_off : 0xFFFFFFFFu, 0, 2);   // nontemporal: written once, not read again here
             }
         }
     }
     if (!nxt.valid) break;
+    stores_behind = prefetched && wave_active && MODE != 1;
     cur = nxt; cp = ncp;
     }   // tiles
 }
@@ -586,10 +620,6 @@ struct SkinnyCfg {
     static_assert(LDS_BYTES <= 160 * 1024, "LDS");
 };
 
-template <int N> __device__ __forceinline__ void wait_vmcnt() {
-    // s_waitcnt with only vmcnt constrained: vmcnt is split over bits [3:0] and [15:14]
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
-}
 
 template <int BN_, int NSTAGE_, int MODE>
 __global__ __launch_bounds__(256)
