@@ -17,6 +17,7 @@ the split-K workspace is cached per device instead of allocated per call
 branch overwrites them, :570-571).
 """
 import ctypes
+import weakref
 
 import torch
 
@@ -45,6 +46,14 @@ def _is_kmajor(t: torch.Tensor) -> bool:
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 _plan_cache = {}   # (m, n, k) -> workspace bytes the planner asks for
+
+# Operands that passed the checks once: a caller that hands over the same five tensor objects again
+# (a benchmark loop, a layer called every step) skips the dtype / shape / stride checks, which cost more
+# host time than a small GEMM takes on the GPU.  An entry is keyed by the identities and version
+# counters of the tensors (any in-place change of a tensor, its metadata included, bumps the counter)
+# and holds weak references, so a recycled id() cannot alias a dead tensor.
+_CHECKED_MAX = 64
+_checked = {}      # key -> (weakrefs, m, n, k, workspace bytes, device index)
 
 
 def _stream_ptr(device: torch.device) -> int:
@@ -94,6 +103,21 @@ def custom_kernel(data, variant: int = 0, split_k: int = 0):
     the defaults let the library's planner decide.
     """
     a, b, a_scale, b_scale, c = data
+    lib = _lib.load()
+    if variant == 0 and split_k == 0:
+        key = (id(a), a._version, id(b), b._version, id(a_scale), a_scale._version, id(b_scale), b_scale._version, id(c), c._version)
+        hit = _checked.get(key)
+        if hit is not None:
+            refs, m, n, k, need, dev_index = hit
+            if refs[0]() is a and refs[1]() is b and refs[2]() is a_scale and refs[3]() is b_scale and refs[4]() is c:
+                ws_ptr, ws_len = None, 0
+                if need:
+                    ws = _workspace(a.device, need)
+                    ws_ptr, ws_len = ws.data_ptr(), ws.numel()
+                if dev_index == torch.cuda.current_device():
+                    _lib.check(lib.fp8bs_gemm_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(), c.data_ptr(),
+                                                 ws_ptr, ws_len, m, n, k, 0, 0, _stream_ptr(a.device)))
+                    return c
     m, k = a.shape
     n = b.shape[0]
     _check_operands(a, b, a_scale, b_scale, c, m, n, k)
@@ -102,12 +126,15 @@ def custom_kernel(data, variant: int = 0, split_k: int = 0):
         raise ValueError("b / b_scale shapes do not match [n, k] / [ceil(n/128), k/128]")
     if not _is_kmajor(b) or not _is_kmajor(b_scale):
         raise ValueError("b and b_scale must be K-major (stride (1, n) / (1, ceil(n/128)))")
-    lib = _lib.load()
     if variant == 0 and split_k == 0:
         need = _plan_cache.get((m, n, k))
         if need is None:
             need = workspace_bytes(m, n, k) if (m > 0 and n > 0 and k > 0) else 0
             _plan_cache[(m, n, k)] = need
+        if len(_checked) >= _CHECKED_MAX:
+            _checked.pop(next(iter(_checked)))
+        _checked[(id(a), a._version, id(b), b._version, id(a_scale), a_scale._version, id(b_scale), b_scale._version, id(c), c._version)] = (
+            tuple(weakref.ref(t) for t in (a, b, a_scale, b_scale, c)), m, n, k, need, a.device.index)
     else:
         need = max(split_k, 1) * m * n * 4 if split_k > 1 else 0
     ws_ptr, ws_len = None, 0

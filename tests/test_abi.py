@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol(pkg):
 def test_plan_shape_families(pkg):
     p = pkg.plan(4096, 4096, 4096)
     assert p.variant == 2 and (p.tile_m, p.tile_n) == (256, 256) and p.split_k == 1 and p.workspace_bytes == 0
-    assert p.grid_x == 256 and p.block_threads == 512 and p.lds_bytes == 2 * (128 * 512 + 1024)
+    assert p.grid_x == 256 and p.block_threads == 512 and p.lds_bytes == 2 * (128 * 512 + 1024 + 256)     # A + B + a_scale row + b_scale values, two stages
     p = pkg.plan(64, 18432, 7168)                       # skinny-M: streaming tile, split-K fills the CUs
     assert p.variant == 6 and (p.tile_m, p.tile_n) == (64, 144) and p.split_k == 2 and p.grid_x == 256
     assert p.workspace_bytes == p.split_k * 64 * 18432 * 4 == pkg.workspace_bytes(64, 18432, 7168)
