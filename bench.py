@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM/fabric bytes per launch of the 256x256 kernel on configuration 2, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch: 49,770 and 32,770) scaled by what the same counters read for a 128 MiB
 # device copy (`--calibrate-copy`: x2.00 and x1.00); the summary is profiles/gemm_tr_256x256_cfg2_4096cubed.txt
-TRAFFIC_CFG2_BYTES = (49769 * 2.00 + 32768 * 1.00) * 1024
+TRAFFIC_CFG2_BYTES = (49779 * 2.00 + 32783 * 1.00) * 1024
 
 
 def algorithmic_bytes(m, n, k):
