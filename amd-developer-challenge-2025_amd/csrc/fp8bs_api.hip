@@ -66,7 +66,21 @@ bool vector_shape(int m, int n) { return (m % 4) == 0 && (n % 8) == 0; }
 // small cost model.  m <= 128 -> the streaming kernel with the K split that fills the CUs.
 void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     if (num_cus <= 0) num_cus = 256;
-    if (!vector_shape(m, n)) { fill_plan(m, n, k, FP8BS_VARIANT_GENERIC, 1, out); return; }
+    if (!vector_shape(m, n)) {
+        // m not a multiple of 4: the planned kernel takes the first m - m % 4 rows (reading a with its
+        // true row length) and a second launch of the streaming kernel the last four rows (a window that
+        // ends exactly at the end of every k row, so the last dword of a is never cut by the buffer's
+        // range check).  The plan describes the first launch; the workspace covers both.
+        if ((n % 8) == 0 && (m & ~3) > 0) {
+            fp8bs_plan_t tail{};
+            choose(m & ~3, n, k, num_cus, out);
+            choose(4, n, k, num_cus, &tail);
+            if (tail.workspace_bytes > out->workspace_bytes) out->workspace_bytes = tail.workspace_bytes;
+            return;
+        }
+        fill_plan(m, n, k, FP8BS_VARIANT_GENERIC, 1, out);
+        return;
+    }
     int kbt = k / KBLK;
     if (m > 128) {
         // Compute-bound family: the tile shape and K split that finish soonest under a cost model in
@@ -186,21 +200,23 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
         if (variant != FP8BS_VARIANT_AUTO && variant != FP8BS_VARIANT_GENERIC) return FP8BS_ERR_BAD_VARIANT;
         variant = FP8BS_VARIANT_GENERIC;
     }
+    int m_main = m;                                    // rows the planned kernel computes
     if (variant == FP8BS_VARIANT_AUTO) {
         choose(m, n, k, 0, &plan);
-        if (split_k > 0) fill_plan(m, n, k, plan.variant, split_k, &plan);
+        if (plan.variant != FP8BS_VARIANT_GENERIC && (m % 4) != 0) m_main = m & ~3;
+        if (split_k > 0) fill_plan(m_main, n, k, plan.variant, split_k, &plan);
     } else {
         VariantInfo vi{};
         if (!variant_info(variant, &vi)) return FP8BS_ERR_BAD_VARIANT;
         if (variant != FP8BS_VARIANT_GENERIC && !vector_shape(m, n)) return FP8BS_ERR_BAD_VARIANT;
         fill_plan(m, n, k, variant, split_k > 0 ? split_k : 1, &plan);
     }
-    if (plan.split_k > 1 && (!ws || ws_bytes < plan.workspace_bytes)) return FP8BS_ERR_WORKSPACE;
+    if (plan.split_k > 1 && (!ws || ws_bytes < (uint64_t)plan.split_k * (uint64_t)m_main * (uint64_t)n * 4u)) return FP8BS_ERR_WORKSPACE;
 
     fp8bs::GemmArgs g{};
     g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.as = a_scale; g.bs = b_scale;
     g.c = (uint16_t*)c; g.ws = (float*)ws; g.row_offsets = nullptr;
-    g.m = m; g.n = n; g.k = k; g.lda = m; g.nb = (n + 127) / 128;
+    g.m = m_main; g.n = n; g.k = k; g.lda = m; g.nb = (n + 127) / 128;
     g.split_k = plan.split_k;
     g.kb_per_split = (int)cdiv(k / KBLK, plan.split_k);
     g.band_h = 4;
@@ -208,7 +224,20 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
     int mode = plan.split_k > 1 ? 1 : 0;
     if (fp8bs::launch_gemm(plan.variant, mode, g, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
     if (mode == 1) {
-        if (fp8bs::launch_splitk_reduce(g.ws, g.c, (size_t)m * n, plan.split_k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
+        if (fp8bs::launch_splitk_reduce(g.ws, g.c, (size_t)m_main * n, plan.split_k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
+    }
+    if (m_main < m) {
+        // the last four rows (one to three of them new): same operands, shifted to row m - 4; the
+        // workspace is free again once the launches above have been queued on the same stream
+        fp8bs_plan_t tp{};
+        choose(4, n, k, 0, &tp);
+        if (tp.split_k > 1 && (!ws || ws_bytes < tp.workspace_bytes)) fill_plan(4, n, k, tp.variant, 1, &tp);
+        fp8bs::GemmArgs t = g;
+        t.a += m - 4; t.as += m - 4; t.c += (size_t)(m - 4) * n; t.row0 = m - 4;
+        t.m = 4; t.split_k = tp.split_k; t.kb_per_split = (int)cdiv(k / KBLK, tp.split_k);
+        const int tmode = tp.split_k > 1 ? 1 : 0;
+        if (fp8bs::launch_gemm(tp.variant, tmode, t, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
+        if (tmode == 1 && fp8bs::launch_splitk_reduce(t.ws, t.c, (size_t)4 * n, tp.split_k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
     }
     return FP8BS_OK;
 }

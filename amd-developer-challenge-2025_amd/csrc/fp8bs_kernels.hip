@@ -244,7 +244,7 @@ void gemm_tr_kernel(const GemmArgs p) {
     };
 
     // ---- buffer resources: out-of-range lanes read zeros instead of faulting -------------------
-    const uint32_t a_bytes = (uint32_t)p.k * (uint32_t)p.lda;
+    const uint32_t a_bytes = (uint32_t)p.k * (uint32_t)p.lda - (uint32_t)p.row0;
     const uint32_t b_bytes = (uint32_t)p.k * (uint32_t)p.n;
     __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, a_bytes, 0x00020000);
 
@@ -293,7 +293,8 @@ void gemm_tr_kernel(const GemmArgs p) {
         c.kb_begin = t.kb_begin;
         c.b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.bptr, 0, b_bytes, 0x00020000);
         c.sc_rsrc = __builtin_amdgcn_make_buffer_rsrc(sc_is_b ? (void*)t.bsptr : (void*)p.as, 0,
-                                                      (uint32_t)(p.k / KBLK) * (sc_is_b ? (uint32_t)p.nb : (uint32_t)p.lda) * 4u, 0x00020000);
+                                                      sc_is_b ? (uint32_t)(p.k / KBLK) * (uint32_t)p.nb * 4u
+                                                              : ((uint32_t)(p.k / KBLK) * (uint32_t)p.lda - (uint32_t)p.row0) * 4u, 0x00020000);
         return c;
     };
     const uint32_t a_kstep = (uint32_t)KBLK * (uint32_t)p.lda, b_kstep = (uint32_t)KBLK * (uint32_t)p.n;
@@ -643,8 +644,8 @@ void gemm_skinny_kernel(const GemmArgs p) {
     const int nkb = kb_end - kb_begin;
     const int nb0 = n0 / 128;
 
-    const uint32_t a_bytes = (uint32_t)p.k * (uint32_t)p.lda, b_bytes = (uint32_t)p.k * (uint32_t)p.n;
-    const uint32_t as_bytes = (uint32_t)kbt * (uint32_t)p.lda * 4u, bs_bytes = (uint32_t)kbt * (uint32_t)p.nb * 4u;
+    const uint32_t a_bytes = (uint32_t)p.k * (uint32_t)p.lda - (uint32_t)p.row0, b_bytes = (uint32_t)p.k * (uint32_t)p.n;
+    const uint32_t as_bytes = ((uint32_t)kbt * (uint32_t)p.lda - (uint32_t)p.row0) * 4u, bs_bytes = (uint32_t)kbt * (uint32_t)p.nb * 4u;
 
     // ---- copy plan.  The one-KiB copies of a block are numbered I = 4q + wave, q = 0..COPIES-1:
     //      I < A_COPIES the A tile, then B_COPIES of the B tile (copy Ib fills B chunks 64*Ib ..), then the

@@ -32,8 +32,11 @@ def test_plan_shape_families(pkg):
     p = pkg.plan(64, 18432, 7168)                       # skinny-M: streaming tile, split-K fills the CUs
     assert p.variant == 6 and (p.tile_m, p.tile_n) == (64, 144) and p.split_k == 2 and p.grid_x == 256
     assert p.workspace_bytes == p.split_k * 64 * 18432 * 4 == pkg.workspace_bytes(64, 18432, 7168)
-    p = pkg.plan(130, 192, 256)                         # not a multiple of 16 -> generic kernel
+    p = pkg.plan(130, 190, 256)                         # n not a multiple of 8 -> generic kernel
     assert p.variant == 1 and p.split_k == 1
+    p, q = pkg.plan(130, 192, 256), pkg.plan(128, 192, 256)   # m % 4 != 0: the plan of the first 128 rows
+    assert p.variant == q.variant != 1 and p.split_k == q.split_k and p.workspace_bytes == q.workspace_bytes
+    assert pkg.plan(3, 192, 256).variant == 1           # fewer than 4 rows: nothing for the vector kernels
     p = pkg.plan(256, 512, 1024)                        # small: one of the sub-256 tiles, never the scalar kernel
     assert p.variant in (3, 4, 5) and p.split_k >= 1 and p.split_k <= 8
     p = pkg.plan(1024, 512, 7168)                       # few tiles, long K: the planner splits K
