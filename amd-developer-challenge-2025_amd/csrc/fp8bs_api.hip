@@ -57,6 +57,9 @@ void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out)
     out->workspace_bytes = split_k > 1 ? (uint64_t)split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
 }
 
+// Bytes at the head of the workspace for the four-row copies of a and a_scale (m < 4).
+uint64_t pad4_bytes(int k) { return (((uint64_t)k * 4u + (uint64_t)(k / KBLK) * 16u) + 255u) & ~(uint64_t)255u; }
+
 // What the vector kernels need of a shape: rows of a (m bytes) that keep the 4-byte loads of a copy
 // aligned and inside the buffer's per-dword range check, rows of c (n bf16) that keep 16-byte stores
 // aligned.
@@ -76,6 +79,13 @@ void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
             choose(m & ~3, n, k, num_cus, out);
             choose(4, n, k, num_cus, &tail);
             if (tail.workspace_bytes > out->workspace_bytes) out->workspace_bytes = tail.workspace_bytes;
+            return;
+        }
+        // one to three rows (a few tokens of a decode step): the operands are copied into four-row
+        // matrices at the head of the workspace and the streaming kernel runs on those
+        if ((n % 8) == 0 && m < 4) {
+            choose(4, n, k, num_cus, out);
+            out->workspace_bytes += pad4_bytes(k);
             return;
         }
         fill_plan(m, n, k, FP8BS_VARIANT_GENERIC, 1, out);
@@ -201,6 +211,28 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
         variant = FP8BS_VARIANT_GENERIC;
     }
     int m_main = m;                                    // rows the planned kernel computes
+    if (variant == FP8BS_VARIANT_AUTO && split_k == 0 && m < 4 && (n % 8) == 0 && k > 0) {
+        // one to three rows: four-row copies of a / a_scale at the head of the workspace, then the
+        // streaming kernel; without enough workspace the generic kernel below does it
+        choose(4, n, k, 0, &plan);
+        const uint64_t pad = pad4_bytes(k);
+        const uint64_t planes = plan.split_k > 1 ? (uint64_t)plan.split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
+        if (ws && ws_bytes >= pad + planes) {
+            uint8_t* a4 = (uint8_t*)ws;
+            float* as4 = (float*)(a4 + (size_t)k * 4);
+            if (fp8bs::launch_pad_rows4((const uint8_t*)a, a_scale, a4, as4, m, k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
+            fp8bs::GemmArgs g{};
+            g.a = a4; g.b = (const uint8_t*)b; g.as = as4; g.bs = b_scale;
+            g.c = (uint16_t*)c; g.ws = (float*)((uint8_t*)ws + pad); g.row_offsets = nullptr;
+            g.m = m; g.n = n; g.k = k; g.lda = 4; g.nb = (n + 127) / 128;
+            g.split_k = plan.split_k; g.kb_per_split = (int)cdiv(k / KBLK, plan.split_k); g.band_h = 4;
+            const int mode = plan.split_k > 1 ? 1 : 0;
+            if (fp8bs::launch_gemm(plan.variant, mode, g, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
+            if (mode == 1 && fp8bs::launch_splitk_reduce(g.ws, g.c, (size_t)m * n, plan.split_k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
+            return FP8BS_OK;
+        }
+        variant = FP8BS_VARIANT_GENERIC;
+    }
     if (variant == FP8BS_VARIANT_AUTO) {
         choose(m, n, k, 0, &plan);
         if (plan.variant != FP8BS_VARIANT_GENERIC && (m % 4) != 0) m_main = m & ~3;

@@ -948,6 +948,25 @@ hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t str
     }
 }
 
+// Fewer than four rows of a (one to three tokens): copy a and a_scale into four-row matrices (rows beyond
+// m are zero).  With four bytes per k row every load of the vector kernels stays on a dword of its own.
+__global__ __launch_bounds__(256)
+void pad_rows4_kernel(const uint8_t* __restrict__ a, const float* __restrict__ as, uint8_t* __restrict__ a4, float* __restrict__ as4, int m, int k) {
+    const int kk = blockIdx.x * 256 + threadIdx.x;
+    if (kk < k) {
+        uint32_t w = 0;
+        for (int i = 0; i < m; i++) w |= (uint32_t)a[(size_t)kk * m + i] << (8 * i);
+        *(uint32_t*)(a4 + 4 * (size_t)kk) = w;
+    }
+    if (kk < k / KBLK)
+        for (int i = 0; i < 4; i++) as4[4 * (size_t)kk + i] = i < m ? as[(size_t)kk * m + i] : 0.f;
+}
+
+hipError_t launch_pad_rows4(const uint8_t* a, const float* as, uint8_t* a4, float* as4, int m, int k, hipStream_t stream) {
+    hipLaunchKernelGGL(pad_rows4_kernel, dim3((unsigned)((k + 255) / 256)), dim3(256), 0, stream, a, as, a4, as4, m, k);
+    return hipGetLastError();
+}
+
 hipError_t launch_splitk_reduce(const float* ws, uint16_t* c, size_t mn, int split_k, hipStream_t stream) {
     size_t threads = (mn + 7) / 8;
     unsigned blocks = (unsigned)((threads + 255) / 256);

@@ -36,7 +36,9 @@ def test_plan_shape_families(pkg):
     assert p.variant == 1 and p.split_k == 1
     p, q = pkg.plan(130, 192, 256), pkg.plan(128, 192, 256)   # m % 4 != 0: the plan of the first 128 rows
     assert p.variant == q.variant != 1 and p.split_k == q.split_k and p.workspace_bytes == q.workspace_bytes
-    assert pkg.plan(3, 192, 256).variant == 1           # fewer than 4 rows: nothing for the vector kernels
+    p, q = pkg.plan(3, 192, 256), pkg.plan(4, 192, 256)       # 1..3 rows: four-row copies in the workspace
+    assert p.variant == q.variant != 1 and p.workspace_bytes == q.workspace_bytes + 1280   # 4*256 + 16*2 -> 1280
+    assert pkg.plan(3, 190, 256).variant == 1
     p = pkg.plan(256, 512, 1024)                        # small: one of the sub-256 tiles, never the scalar kernel
     assert p.variant in (3, 4, 5) and p.split_k >= 1 and p.split_k <= 8
     p = pkg.plan(1024, 512, 7168)                       # few tiles, long K: the planner splits K

@@ -79,7 +79,8 @@ def test_every_variant_and_split_on_config1(pkg, oracle, dev, variant, split_k):
 @pytest.mark.parametrize("m,n,k", [(16, 16, 128), (48, 80, 128), (272, 2112, 512), (256, 256, 256), (304, 400, 384),
                                    (64, 1024, 1024), (512, 144, 1280), (130, 192, 256), (1, 7, 128), (33, 129, 384),
                                    (132, 200, 256), (20, 24, 128), (516, 264, 384), (268, 2104, 256),
-                                   (4095, 512, 256), (1021, 264, 384), (131, 1024, 512), (61, 2048, 1024), (5, 16, 128)])
+                                   (4095, 512, 256), (1021, 264, 384), (131, 1024, 512), (61, 2048, 1024), (5, 16, 128),
+                                   (1, 2048, 1024), (2, 264, 384), (3, 18432, 512)])
 def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
     """N tails (2112 = 16*128 + 64), tiles larger than the matrix, rows and columns that end inside a
     16-byte chunk (m % 4 == 0, n % 8 == 0: still the vector kernels), shapes only the generic kernel takes."""
@@ -87,8 +88,8 @@ def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
     cpu = pkg.inputs.make_dense(cfg, m=m, n=n, k=k)
     out = pkg.custom_kernel(_to(cpu, dev))
     _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d" % (m, n, k))
-    if n % 8 == 0 and m >= 4:
-        assert pkg.plan(m, n, k).variant != 1                   # odd m: vector kernels + 1..3 rows on the generic one
+    if n % 8 == 0:
+        assert pkg.plan(m, n, k).variant != 1                   # any m: the vector kernels, in two launches if m % 4 != 0
     if m % 4 == 0 and n % 8 == 0:
         for variant in (2, 3, 4, 5, 6, 7, 8):
             out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1)
