@@ -102,7 +102,7 @@ __device__ __forceinline__ void band_tile(int v, int tiles_m, int tiles_n, int g
 //   MODE 2  : grouped (row_offsets), bf16 output
 // LDS: 2 stages, each [128 k][BM] bytes of A then [128 k][BN] bytes of B, 16-byte chunks XOR-swizzled
 // so that the 16 k rows touched by half a wave in one transposing read fall on 16 different 16-byte
-// bank groups.
+// bank groups, then the k block's a_scale row and b_scale values.
 // ---------------------------------------------------------------------------------------------------
 template <int BM, int BN, int WM, int WN, int MODE>
 struct TileCfg {
