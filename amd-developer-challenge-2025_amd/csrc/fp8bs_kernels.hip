@@ -364,8 +364,9 @@ void gemm_tr_kernel(const GemmArgs p) {
     const int row_lo = cur.row_lo, row_hi = cur.row_hi;
     // a_scale: lane's output row of m-tile t is tile row wave_m*WM + 16t + i16, read from the stage's
     // copy of the a_scale row.
-    // does any row of this wave's tile get stored?
-    const bool wave_active = __builtin_amdgcn_readfirstlane((m0 + wave_m * WM < row_hi && m0 + wave_m * WM + WM > row_lo) ? 1 : 0) != 0;
+    // does any element of this wave's tile get stored?  (rows of the expert / matrix, columns of the matrix)
+    const bool wave_active = __builtin_amdgcn_readfirstlane((m0 + wave_m * WM < row_hi && m0 + wave_m * WM + WM > row_lo &&
+                                                             n0 + wave_n * WN < p.n) ? 1 : 0) != 0;
 
     v4f acc[C::MT][C::NT];
 #pragma unroll
