@@ -96,6 +96,27 @@ def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
             _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d" % (m, n, k, variant))
 
 
+@pytest.mark.parametrize("m,n,k,variant", [(8192, 8192, 256, 2), (8188, 4104, 128, 0), (4096, 8192, 384, 5),
+                                           (8192, 4096, 256, 3), (4096, 4096, 256, 4)])
+def test_many_tiles_per_workgroup_against_the_scalar_kernel(pkg, oracle, dev, m, n, k, variant):
+    """Short K and a large output: every persistent workgroup walks many tiles, so the hand-over between
+    tiles (next tile's first block issued ahead of the output stores, counted wait) carries the result.
+    Every element is compared with the scalar HIP kernel on the same operands."""
+    cfg = pkg.inputs.CONFIGS[2]
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randint(0, 0x78, (k, m), dtype=torch.uint8, generator=g) | (torch.randint(0, 2, (k, m), dtype=torch.uint8, generator=g) << 7)
+    b = torch.randint(0, 0x78, (k, n), dtype=torch.uint8, generator=g) | (torch.randint(0, 2, (k, n), dtype=torch.uint8, generator=g) << 7)
+    a_scale = (torch.rand(k // 128, m, generator=g) + 0.5) * 1e-3
+    b_scale = (torch.rand(k // 128, (n + 127) // 128, generator=g) + 0.5) * 1e-3
+    data = (a.to(dev).view(torch.float8_e4m3fn).t(), b.to(dev).view(torch.float8_e4m3fn).t(), a_scale.to(dev).t(), b_scale.to(dev).t())
+    c1 = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    c2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+    ref = pkg.custom_kernel(data + (c1,), variant=1, split_k=1).float()
+    out = pkg.custom_kernel(data + (c2,), variant=variant, split_k=1 if variant else 0).float()
+    bad = ~((out - ref).abs() <= ATOL + RTOL * ref.abs())
+    assert int(bad.sum()) == 0, "%d elements differ, first at %s" % (int(bad.sum()), bad.nonzero()[0].tolist())
+
+
 def test_repeated_calls_skip_the_checks_but_not_after_a_change(pkg, oracle, dev):
     """The second call with the same tensor objects takes the short path; a tensor changed in place, or
     another tensor object of a wrong layout, is checked again."""
