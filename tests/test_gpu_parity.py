@@ -291,6 +291,23 @@ def test_grouped_full_size_sampled_rows(pkg, oracle, dev):
     _check(oracle, out[rows.to(dev)], oracle.ref_grouped(cpu, rows=rows), "config 5 sampled rows")
 
 
+def test_grouped_every_element_against_the_scalar_kernel(pkg, dev):
+    """Configuration 5's routing and shapes with K = 256: ~2300 tiles over 256 persistent workgroups.  The
+    whole output is compared with the scalar kernel's (taken by handing over a c that starts off the
+    16-byte grid)."""
+    cfg = pkg.inputs.CONFIGS[4]
+    data = list(_to(pkg.inputs.make_grouped(cfg, k=256), dev))
+    data[5].fill_(float("nan"))
+    out = pkg.grouped_kernel(tuple(data)).float()
+    scalar = list(data)
+    scalar[5] = _shifted(torch.full_like(data[5], float("nan")), 2)
+    assert scalar[5].data_ptr() % 16 != 0
+    ref = pkg.grouped_kernel(tuple(scalar)).float()
+    assert not bool(ref.isnan().any()) and not bool(out.isnan().any())
+    bad = ~((out - ref).abs() <= ATOL + RTOL * ref.abs())
+    assert int(bad.sum()) == 0, "%d elements differ, first at %s" % (int(bad.sum()), bad.nonzero()[0].tolist())
+
+
 def test_special_codes(pkg, oracle, dev):
     """-0, the largest codes (+-448), the smallest subnormals and NaN codes: a NaN in a row of A or B
     poisons exactly the outputs that row takes part in, everything else stays within the bar."""
