@@ -623,7 +623,10 @@ struct SkinnyCfg {
 };
 
 
-template <int BN_, int NSTAGE_, int MODE>
+// MTV: the 16-row m tiles that get multiplied, 1..4.  Fewer than 4 only when the whole matrix has at
+// most 16*MTV rows (a decode step has one to a few): a compile-time count, because a run-time test per
+// m tile put branches between the MFMAs and their folds, and results read back too early were seen.
+template <int BN_, int NSTAGE_, int MODE, int MTV>
 __global__ __launch_bounds__(256)
 void gemm_skinny_kernel(const GemmArgs p) {
     using C = SkinnyCfg<BN_, NSTAGE_>;
@@ -684,7 +687,8 @@ void gemm_skinny_kernel(const GemmArgs p) {
     // All copies of K block `blk` (relative to kb_begin).  Beyond the last block the same number of
     // copies is issued against empty buffers (every lane out of range: zeros land in a free stage and no
     // memory is read), which keeps the count of outstanding copies per wave the same in every iteration.
-    auto issue_block = [&](int blk) {
+    auto issue_block = [&](auto wave_tag, int blk) {
+        constexpr int W = decltype(wave_tag)::value;
         const uint32_t st = lds_base + (uint32_t)(blk % C::NSTAGE) * C::STAGE_BYTES;
         const bool live = blk < nkb;
         const uint32_t kb = (uint32_t)(kb_begin + (live ? blk : 0));
@@ -693,14 +697,15 @@ void gemm_skinny_kernel(const GemmArgs p) {
         __amdgpu_buffer_rsrc_t as_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.as, 0, live ? as_bytes : 0u, 0x00020000);
         __amdgpu_buffer_rsrc_t bs_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.bs, 0, live ? bs_bytes : 0u, 0x00020000);
         const uint32_t a_k = kb * (uint32_t)KBLK * (uint32_t)p.lda, b_k = kb * (uint32_t)KBLK * (uint32_t)p.n;
-#pragma unroll
-        for (int q = 0; q < C::COPIES; q++) {
-            const int I = 4 * q + wave;          // wave-uniform
-            if (I < C::A_COPIES) copy16_global_to_lds(a_rsrc, st + I * 1024, voff[q], a_k);
-            else if (I < C::A_COPIES + C::B_COPIES) copy16_global_to_lds(b_rsrc, st + C::A_BYTES + (I - C::A_COPIES) * 1024, voff[q], b_k);
-            else if (I == C::A_COPIES + C::B_COPIES) copy4_global_to_lds(as_rsrc, st + C::A_BYTES + C::B_BYTES, voff[q], kb * (uint32_t)p.lda * 4u);
-            else copy4_global_to_lds(bs_rsrc, st + C::A_BYTES + C::B_BYTES + 256, voff[q], kb * (uint32_t)p.nb * 4u);
-        }
+        [&]<int... Q>(std::integer_sequence<int, Q...>) {
+            ([&] {
+                constexpr int I = 4 * Q + W;
+                if constexpr (I < C::A_COPIES) copy16_global_to_lds(a_rsrc, st + I * 1024, voff[Q], a_k);
+                else if constexpr (I < C::A_COPIES + C::B_COPIES) copy16_global_to_lds(b_rsrc, st + C::A_BYTES + (I - C::A_COPIES) * 1024, voff[Q], b_k);
+                else if constexpr (I == C::A_COPIES + C::B_COPIES) copy4_global_to_lds(as_rsrc, st + C::A_BYTES + C::B_BYTES, voff[Q], kb * (uint32_t)p.lda * 4u);
+                else copy4_global_to_lds(bs_rsrc, st + C::A_BYTES + C::B_BYTES + 256, voff[Q], kb * (uint32_t)p.nb * 4u);
+            }(), ...);
+        }(std::make_integer_sequence<int, C::COPIES>{});
     };
 
     // ---- LDS read addresses ----
@@ -716,14 +721,18 @@ void gemm_skinny_kernel(const GemmArgs p) {
 #pragma unroll
         for (int x = 0; x < C::NT_MAX; x++) acc[t][x] = (v4f){0.f, 0.f, 0.f, 0.f};
 
+    // The loop is instantiated once per wave index: which copies a wave issues and which n tiles it
+    // multiplies then are compile-time facts, and the loop body has no branches.
+    auto k_loop = [&](auto wave_tag) {
+    constexpr int W = decltype(wave_tag)::value;
     // ---- prologue: NSTAGE-1 blocks in flight ----
-    for (int b = 0; b < C::NSTAGE - 1; b++) issue_block(b);
+    for (int b = 0; b < C::NSTAGE - 1; b++) issue_block(wave_tag, b);
 
     for (int j = 0; j < nkb; j++) {
         // the NSTAGE-2 blocks issued after block j may still be on their way
         wait_vmcnt<(C::NSTAGE - 2) * C::COPIES>();
         __syncthreads();      // block j complete in LDS; everyone is done with the stage of block j-1
-        issue_block(j + C::NSTAGE - 1);
+        issue_block(wave_tag, j + C::NSTAGE - 1);
 
         const unsigned char* sbase = lds + (j % C::NSTAGE) * C::STAGE_BYTES;
         const unsigned char* sc = sbase + C::A_BYTES + C::B_BYTES;
@@ -731,18 +740,20 @@ void gemm_skinny_kernel(const GemmArgs p) {
         v8i areg[C::MT];
 #pragma unroll
         for (int t = 0; t < C::MT; t++) {
-            asv[t] = *(const float*)(sc + (16 * t + i16) * 4);
-            const unsigned char* q = sbase + a_lane_off + ((t ^ swz_a) << 4);
+            if (t < MTV) {                               // m tiles beyond the matrix do no work
+                asv[t] = *(const float*)(sc + (16 * t + i16) * 4);
+                const unsigned char* q = sbase + a_lane_off + ((t ^ swz_a) << 4);
 #pragma unroll
-            for (int jj = 0; jj < 4; jj++) {
-                v2i x = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_V2I(q + jj * 32 * C::BM));
-                areg[t][2 * jj] = x[0]; areg[t][2 * jj + 1] = x[1];
+                for (int jj = 0; jj < 4; jj++) {
+                    v2i x = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_V2I(q + jj * 32 * C::BM));
+                    areg[t][2 * jj] = x[0]; areg[t][2 * jj + 1] = x[1];
+                }
             }
         }
-#pragma unroll
-        for (int x = 0; x < C::NT_MAX; x++) {
-            const int u = wave + 4 * x;                 // wave-uniform
-            if (u < C::CPR_B) {
+        [&]<int... X>(std::integer_sequence<int, X...>) {
+            ([&] {
+            constexpr int x = X, u = W + 4 * X;
+            if constexpr (u < C::CPR_B) {
                 v8i breg;
                 const unsigned char* q = sbase + b_lane_off + ((u ^ swz_b) << 4);
 #pragma unroll
@@ -754,14 +765,24 @@ void gemm_skinny_kernel(const GemmArgs p) {
                 const float bsv = *(const float*)(sc + 256 + bi * 4);
 #pragma unroll
                 for (int t = 0; t < C::MT; t++) {
-                    const v4f z = {0.f, 0.f, 0.f, 0.f};
-                    v4f d = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(breg, areg[t], z, 0, 0, 0, 0, 0, 0);
-                    const float s = asv[t] * bsv;
+                    if (t < MTV) {
+                        const v4f z = {0.f, 0.f, 0.f, 0.f};
+                        v4f d = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(breg, areg[t], z, 0, 0, 0, 0, 0, 0);
+                        const float s = asv[t] * bsv;
 #pragma unroll
-                    for (int r = 0; r < 4; r++) acc[t][x][r] = __builtin_fmaf(d[r], s, acc[t][x][r]);
+                        for (int r = 0; r < 4; r++) acc[t][x][r] = __builtin_fmaf(d[r], s, acc[t][x][r]);
+                    }
                 }
             }
-        }
+            }(), ...);
+        }(std::make_integer_sequence<int, C::NT_MAX>{});
+    }
+    };   // k_loop
+    switch (wave) {
+        case 0: k_loop(std::integral_constant<int, 0>{}); break;
+        case 1: k_loop(std::integral_constant<int, 1>{}); break;
+        case 2: k_loop(std::integral_constant<int, 2>{}); break;
+        default: k_loop(std::integral_constant<int, 3>{}); break;
     }
 
     wait_vmcnt<0>();          // the trailing empty copies still target this workgroup's LDS
@@ -920,14 +941,29 @@ template <int BN, int NSTAGE>
 static hipError_t launch_skinny(const GemmArgs& a, int mode, hipStream_t stream) {
     if (mode == 2 || a.epi != 0) return hipErrorInvalidValue;
     using C = SkinnyCfg<BN, NSTAGE>;
-    auto k0 = gemm_skinny_kernel<BN, NSTAGE, 0>;
-    auto k1 = gemm_skinny_kernel<BN, NSTAGE, 1>;
-    static int raised0[MAX_DEVICES], raised1[MAX_DEVICES];
-    hipError_t e = mode == 1 ? raise_lds_limit((const void*)k1, C::LDS_BYTES, raised1) : raise_lds_limit((const void*)k0, C::LDS_BYTES, raised0);
+    // m tiles with rows: fewer than 4 only for the planner's tile width and a matrix of at most 48 rows
+    const int mtv = (BN == 144 && a.m <= 48) ? (a.m + 15) / 16 : 4;
+    void (*kern)(const GemmArgs) = nullptr;
+    if (mode == 1) {
+        kern = gemm_skinny_kernel<BN, NSTAGE, 1, 4>;
+        if constexpr (BN == 144) {
+            if (mtv == 1) kern = gemm_skinny_kernel<BN, NSTAGE, 1, 1>;
+            if (mtv == 2) kern = gemm_skinny_kernel<BN, NSTAGE, 1, 2>;
+            if (mtv == 3) kern = gemm_skinny_kernel<BN, NSTAGE, 1, 3>;
+        }
+    } else {
+        kern = gemm_skinny_kernel<BN, NSTAGE, 0, 4>;
+        if constexpr (BN == 144) {
+            if (mtv == 1) kern = gemm_skinny_kernel<BN, NSTAGE, 0, 1>;
+            if (mtv == 2) kern = gemm_skinny_kernel<BN, NSTAGE, 0, 2>;
+            if (mtv == 3) kern = gemm_skinny_kernel<BN, NSTAGE, 0, 3>;
+        }
+    }
+    static int raised[8][MAX_DEVICES];
+    hipError_t e = raise_lds_limit((const void*)kern, C::LDS_BYTES, raised[(mode == 1 ? 4 : 0) + mtv - 1]);
     if (e != hipSuccess) return e;
     int tiles = ((a.n + C::BN - 1) / C::BN) * a.split_k * ((a.m + C::BM - 1) / C::BM);
-    if (mode == 1) hipLaunchKernelGGL(k1, dim3(tiles), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
-    else hipLaunchKernelGGL(k0, dim3(tiles), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
+    hipLaunchKernelGGL(kern, dim3(tiles), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
     return hipGetLastError();
 }
 
