@@ -187,6 +187,19 @@ def main():
             "name": cfg.name, "us": round(us, 2), "us_min": round(us_min, 2), "tflops": round(tf, 1), "gbs": round(gbs, 1),
             "input_sets": 1 if cfg.experts else nsets, "bound": bound, "frac": round(tf / PEAK_FP8_TFLOPS if bound == "mfma" else gbs / PEAK_HBM_GBS, 4)}
         d = sets = None
+    # ---- a decode step's shape: configuration 4's weight matrix against a single token row ----
+    if 4 in wanted:
+        cfg4 = pkg.inputs.CONFIGS[3]
+        dcfg = pkg.inputs.Config("decode_1x%dx%d" % (cfg4.n, cfg4.k), 1, cfg4.n, cfg4.k, 0.0, 1.0, cfg4.b_std, 0, 0, cfg4.seed + 7)
+        torch.cuda.empty_cache()
+        by = algorithmic_bytes(1, dcfg.n, dcfg.k)
+        nsets = min(8, -(-3 * 256 * 2 ** 20 // by))
+        sets = [gpu_dense_inputs(pkg, dcfg, dev, dcfg.seed + 100 * s) for s in range(nsets)]
+        us, us_min = time_calls(lambda i: pkg.custom_kernel(sets[i % nsets]), args.steps, args.warmup)
+        per_config[dcfg.name] = {"us": round(us, 2), "us_min": round(us_min, 2), "gbs": round(by / us * 1e-3, 1), "bytes": by,
+                                 "input_sets": nsets, "bound": "hbm", "frac": round(by / us * 1e-3 / PEAK_HBM_GBS, 4),
+                                 "note": "one row: a and a_scale copied to four-row matrices, then the streaming kernel"}
+        sets = None
     # ---- the quantisers in front of the GEMM (HBM-bound): activations of configuration 3, one expert's
     # weights of configuration 5; 4 rotating inputs (> 256 MB in total) so that reads come from HBM ----
     if args.quant:
