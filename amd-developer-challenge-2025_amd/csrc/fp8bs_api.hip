@@ -28,6 +28,8 @@ bool variant_info(int variant, VariantInfo* out) {
         case FP8BS_VARIANT_SKINNY64x144: *out = {64, 144, 256}; return true;
         case FP8BS_VARIANT_SKINNY64x256: *out = {64, 256, 256}; return true;
         case FP8BS_VARIANT_SKINNY64x288: *out = {64, 288, 256}; return true;
+        case FP8BS_VARIANT_T256x192: *out = {256, 192, 512}; return true;
+        case FP8BS_VARIANT_T256x128S3: *out = {256, 128, 512}; return true;
         default: return false;
     }
 }
@@ -101,9 +103,10 @@ void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
         // split adds the fp32 partial planes (written and read back, mostly through the 256 MB cache) and the
         // reduce launch.
         struct Cand { int variant; int rmax; double t_block[3], t_fixed[3]; };
-        const Cand cands[4] = {
+        const Cand cands[5] = {
             {FP8BS_VARIANT_T256x256, 1, {1.87, 0, 0}, {6.8, 0, 0}},
-            {FP8BS_VARIANT_T256x128, 1, {1.22, 0, 0}, {4.4, 0, 0}},
+            {FP8BS_VARIANT_T256x192, 1, {1.45, 0, 0}, {6.0, 0, 0}},
+            {FP8BS_VARIANT_T256x128S3, 1, {1.18, 0, 0}, {4.2, 0, 0}},
             {FP8BS_VARIANT_T128x128, 2, {0.89, 1.34, 0}, {3.1, 4.8, 0}},
             {FP8BS_VARIANT_T64x128, 3, {0.70, 1.04, 1.39}, {1.9, 2.3, 3.6}},
         };

@@ -104,8 +104,9 @@ __device__ __forceinline__ void band_tile(int v, int tiles_m, int tiles_n, int g
 // so that the 16 k rows touched by half a wave in one transposing read fall on 16 different 16-byte
 // bank groups, then the k block's a_scale row and b_scale values.
 // ---------------------------------------------------------------------------------------------------
-template <int BM, int BN, int WM, int WN, int MODE>
+template <int BM, int BN, int WM, int WN, int MODE, int NSTAGE_ = 2>
 struct TileCfg {
+    static constexpr int NSTAGE = NSTAGE_;                           // LDS stages of one K block each
     static constexpr int WAVES_M = BM / WM, WAVES_N = BN / WN;
     static constexpr int NWAVES = WAVES_M * WAVES_N;
     static constexpr int NTHREADS = NWAVES * 64;
@@ -116,11 +117,18 @@ struct TileCfg {
     static constexpr int AS_AREA = AS_BYTES < 1024 ? 1024 : AS_BYTES;
     static constexpr int BS_AREA = 256;                              // the k block's b_scale values of the tile's n blocks
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + AS_AREA + BS_AREA;
-    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
+    static_assert(NSTAGE == 2 || NSTAGE == 3, "two or three stages");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS");
     static constexpr int A_LOADS = A_BYTES / 16 / NTHREADS;         // 16-byte loads per thread per block
     static constexpr int B_LOADS = B_BYTES / 16 / NTHREADS;
     static_assert(A_BYTES % (16 * NTHREADS) == 0 && B_BYTES % (16 * NTHREADS) == 0, "tile/threads");
-    static_assert(WN <= 128 && 128 % WN == 0, "a wave's n range must stay inside one b_scale block");
+    // A wave's n range lies inside one b_scale block when the tile starts on a block boundary and the
+    // wave width divides 128.  Otherwise (BN = 192, WN = 96) it may cross one boundary, at an n tile that
+    // depends on the tile and the wave: the K loop is instantiated per boundary position.
+    static constexpr bool SPLIT_SCALES = !(BN % 128 == 0 && 128 % WN == 0);
+    static_assert(WN <= 128, "a wave's n range crosses at most one b_scale block boundary");
+    static_assert(!SPLIT_SCALES || (BN == 192 && WN == 96), "boundary positions are enumerated for the 192-wide tile only");
     static_assert(CPR_A <= 16 && CPR_B <= 16, "swizzle assumes a k row spans at most 256 bytes");
 };
 
@@ -129,11 +137,35 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
+// same, and all LDS and scalar-memory results back (lgkmcnt(0))
+template <int N> __device__ __forceinline__ void wait_vmcnt_lgkm0() {
+    __builtin_amdgcn_s_waitcnt(0x0070 | (N & 15) | ((N >> 4) << 14));
+}
+
 template <int CPR>
 __device__ __forceinline__ int swz_of_krow(int krow) {
-    // rows per 256-byte bank sweep = 16/CPR; consecutive sweeps get consecutive XOR masks
-    constexpr int ROWS_PER_SWEEP = CPR <= 16 ? 16 / CPR : 1;      // (wider rows are never swizzled)
-    return (krow / ROWS_PER_SWEEP) % CPR;
+    if constexpr (CPR != 12) {
+        // rows per 256-byte bank sweep = 16/CPR; consecutive sweeps get consecutive XOR masks
+        constexpr int ROWS_PER_SWEEP = CPR <= 16 ? 16 / CPR : 1;      // (wider rows are never swizzled)
+        return (krow / ROWS_PER_SWEEP) % CPR;
+    } else {
+        // 12 chunks per k row (192 bytes): four consecutive rows start on the four different quarters of
+        // a 256-byte bank sweep, the next four repeat them; rotating the chunks of each group of four
+        // rows by one more position puts any 16 consecutive rows of one chunk column on 16 different
+        // 16-byte bank groups.
+        return (krow >> 2) & 3;
+    }
+}
+// position of logical chunk `ch` inside its k row, and back
+template <int CPR>
+__device__ __forceinline__ int chunk_to_stored(int ch, int swz) {
+    if constexpr ((CPR & (CPR - 1)) == 0) return ch ^ swz;
+    else { int x = ch + swz; return x >= CPR ? x - CPR : x; }
+}
+template <int CPR>
+__device__ __forceinline__ int stored_to_chunk(int st, int swz) {
+    if constexpr ((CPR & (CPR - 1)) == 0) return st ^ swz;
+    else { int x = st - swz; return x < 0 ? x + CPR : x; }
 }
 
 // EPI 0: plain bf16 output.  EPI 1: gate/up pairs - column 2i is gate_i, column 2i+1 is up_i - are
@@ -145,16 +177,18 @@ __device__ __forceinline__ float silu_mul(float gate, float up) {
     return gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * gate)) * up;
 }
 
-template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0>
+template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0, int NSTAGE = 2>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64)
 void gemm_tr_kernel(const GemmArgs p) {
-    using C = TileCfg<BM, BN, WM, WN, MODE>;
+    using C = TileCfg<BM, BN, WM, WN, MODE, NSTAGE>;
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
 
     // global store instructions per wave and tile in the bf16 epilogue (always this many: lanes without
     // a valid element are switched off by an out-of-range buffer offset, not by a branch)
     constexpr int EPI_WNO = EPI == 1 ? WN / 2 : WN;
-    constexpr int EPI_STORES = MODE == 1 ? 0 : 2 * ((WM / 2) * (EPI_WNO * 2 / 16) / 64);
+    constexpr int EPI_ROW_CHUNKS = EPI_WNO * 2 / 16;
+    constexpr int EPI_ROWS_PER_PASS = (EPI_ROW_CHUNKS & (EPI_ROW_CHUNKS - 1)) == 0 ? 64 / EPI_ROW_CHUNKS : 4;
+    constexpr int EPI_STORES = MODE == 1 ? 0 : 2 * ((WM / 2) / EPI_ROWS_PER_PASS);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -265,6 +299,9 @@ void gemm_tr_kernel(const GemmArgs p) {
     // to overlap.  With the scales in LDS the K loop has no loads of its own that the compiler would have
     // to order against the output stores of the previous tile.
     constexpr int ROWS_PER_COPY_A = C::NWAVES * 64 / C::CPR_A, ROWS_PER_COPY_B = C::NWAVES * 64 / C::CPR_B;
+    // With 12 chunks per k row of B one copy of the workgroup (NWAVES*64 chunks) does not end on a row
+    // boundary: a lane's (k row, chunk) then differs from copy to copy and it keeps one offset per copy.
+    constexpr bool B_ROWS_WHOLE = (C::NWAVES * 64) % C::CPR_B == 0;
     constexpr int AS_COPIES = BM / 64;
     static_assert(C::NWAVES > AS_COPIES, "some wave must be left to copy the b_scale values");
     const bool sc_is_b = wave >= AS_COPIES;                       // this wave's scale copy is the b_scale one
@@ -272,6 +309,7 @@ void gemm_tr_kernel(const GemmArgs p) {
     const uint32_t sc_kstep = (sc_is_b ? (uint32_t)p.nb : (uint32_t)p.lda) * 4u;
     struct CopyPlan {
         uint32_t a_voff, b_voff, sc_voff;
+        uint32_t b_voffq[C::B_LOADS];           // only without B_ROWS_WHOLE
         int kb_begin;
         __amdgpu_buffer_rsrc_t b_rsrc, sc_rsrc;
     };
@@ -282,10 +320,21 @@ void gemm_tr_kernel(const GemmArgs p) {
         int col = t.m0 + 16 * ch;
         col = col < p.lda ? col : t.m0;
         c.a_voff = (uint32_t)krow * (uint32_t)p.lda + (uint32_t)col;
-        krow = P / C::CPR_B; ch = (P % C::CPR_B) ^ swz_of_krow<C::CPR_B>(krow);
+        krow = P / C::CPR_B; ch = stored_to_chunk<C::CPR_B>(P % C::CPR_B, swz_of_krow<C::CPR_B>(krow));
         col = t.n0 + 16 * ch;
         col = col < p.n ? col : t.n0;
         c.b_voff = (uint32_t)krow * (uint32_t)p.n + (uint32_t)col;
+#pragma unroll
+        for (int q = 0; q < C::B_LOADS; q++) {
+            c.b_voffq[q] = 0;
+            if constexpr (!B_ROWS_WHOLE) {
+                const int Pq = q * C::NWAVES * 64 + P;
+                const int kr = Pq / C::CPR_B;
+                int cl = t.n0 + 16 * stored_to_chunk<C::CPR_B>(Pq % C::CPR_B, swz_of_krow<C::CPR_B>(kr));
+                cl = cl < p.n ? cl : t.n0;
+                c.b_voffq[q] = (uint32_t)kr * (uint32_t)p.n + (uint32_t)cl;
+            }
+        }
         int r = sc_is_b ? t.n0 / 128 + lane : t.m0 + wave * 64 + lane;      // n block or row of a
         const int last = (sc_is_b ? p.nb : p.lda) - 1;
         r = r < last ? r : last;
@@ -314,7 +363,10 @@ void gemm_tr_kernel(const GemmArgs p) {
             copy16_global_to_lds(a_rsrc, sa + q * C::NWAVES * 1024, cp.a_voff, kb * a_kstep + (uint32_t)(q * ROWS_PER_COPY_A) * (uint32_t)p.lda);
         } else if constexpr (q < C::A_LOADS + C::B_LOADS) {
             constexpr int qb = q - C::A_LOADS;
-            copy16_global_to_lds(cp.b_rsrc, sa + C::A_BYTES + qb * C::NWAVES * 1024, cp.b_voff, kb * b_kstep + (uint32_t)(qb * ROWS_PER_COPY_B) * (uint32_t)p.n);
+            if constexpr (B_ROWS_WHOLE)
+                copy16_global_to_lds(cp.b_rsrc, sa + C::A_BYTES + qb * C::NWAVES * 1024, cp.b_voff, kb * b_kstep + (uint32_t)(qb * ROWS_PER_COPY_B) * (uint32_t)p.n);
+            else
+                copy16_global_to_lds(cp.b_rsrc, sa + C::A_BYTES + qb * C::NWAVES * 1024, cp.b_voffq[qb], kb * b_kstep);
         } else {
             copy4_global_to_lds(cp.sc_rsrc, lds_base + stage * C::STAGE_BYTES + sc_dst, cp.sc_voff, kb * sc_kstep);
         }
@@ -343,7 +395,7 @@ void gemm_tr_kernel(const GemmArgs p) {
         }
     };
     auto read_b = [&](v8i& dst, int u, const unsigned char* sbase) {
-        const unsigned char* q = sbase + b_lane_off + (((b_chunk0 + u) ^ swz_b) << 4);
+        const unsigned char* q = sbase + b_lane_off + (chunk_to_stored<C::CPR_B>(b_chunk0 + u, swz_b) << 4);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             v2i x = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_V2I(q + j * 32 * BN));
@@ -352,7 +404,7 @@ void gemm_tr_kernel(const GemmArgs p) {
     };
 
     const int as_lane_off = C::A_BYTES + C::B_BYTES + (wave_m * WM + i16) * 4;
-    const int bs_off = C::A_BYTES + C::B_BYTES + C::AS_AREA + (wave_n * WN / 128) * 4;   // a wave's n range lies inside one 128-block
+    const int bs_base = C::A_BYTES + C::B_BYTES + C::AS_AREA;     // slot i: b_scale of n block n0/128 + i
 
     Tile cur = pick_tile(0);
     if (!cur.valid) return;
@@ -367,6 +419,10 @@ void gemm_tr_kernel(const GemmArgs p) {
     // does any element of this wave's tile get stored?  (rows of the expert / matrix, columns of the matrix)
     const bool wave_active = __builtin_amdgcn_readfirstlane((m0 + wave_m * WM < row_hi && m0 + wave_m * WM + WM > row_lo &&
                                                              n0 + wave_n * WN < p.n) ? 1 : 0) != 0;
+    // b_scale of the wave's n tiles: slot bs_off for n tiles [0, ub), the next slot for [ub, NT)
+    const int wave_col = (C::SPLIT_SCALES ? (n0 & 127) : 0) + wave_n * WN;               // from the start of the tile's first n block
+    const int bs_off = bs_base + (wave_col >> 7) * 4;
+    const int ub = C::SPLIT_SCALES ? (128 - (wave_col & 127)) >> 4 : C::NT;
 
     v4f acc[C::MT][C::NT];
 #pragma unroll
@@ -386,19 +442,30 @@ void gemm_tr_kernel(const GemmArgs p) {
         constexpr int DMA_EVERY = (STEPS - C::MT) / NL_EARLY >= 2 ? 2 : 1, DMA_FIRST = DMA_EVERY - 1;
         static_assert(NL_EARLY * DMA_EVERY <= STEPS - C::MT, "not enough steps to issue the copies before the barrier");
 
-        // ---- prologue: block 0 -> stage 0 (unless the previous tile already sent it), wait; first
-        //      copies of block 1 -> stage 1.  The barrier also ends the previous tile's use of stage 1
-        //      as the staging area of its output ----
+        // ---- prologue: blocks 0 .. NSTAGE-2 -> stages 0 .. NSTAGE-2 (unless the previous tile already
+        //      sent them), wait for block 0; first copies of block NSTAGE-1 -> the last stage.  The
+        //      barrier also ends the previous tile's use of the last stage as the staging area of its
+        //      output ----
         // The vector memory counter retires loads and stores in the order they were issued.  If block 0
         // was sent ahead of the previous tile's NSTORES output stores, "at most NSTORES outstanding" means
-        // the block has landed, and the stores are left to finish under the first K block.
-        if (!prefetched) issue_all(cp, 0, 0);
-        if (prefetched && stores_behind) wait_vmcnt<EPI_STORES>();
-        else wait_vmcnt<0>();
+        // the block has landed, and the stores are left to finish under the first K block.  With three
+        // stages block 1 (NLOADS copies) sits between block 0 and the stores.
+        if (!prefetched) {
+            issue_all(cp, 0, 0);
+            if constexpr (NSTAGE == 3) { if (nkb > 1) issue_all(cp, 1, 1); }
+        }
+        if constexpr (NSTAGE == 2) {
+            if (prefetched && stores_behind) wait_vmcnt<EPI_STORES>();
+            else wait_vmcnt<0>();
+        } else {
+            const bool sb = prefetched && stores_behind;
+            if (nkb > 1) { if (sb) wait_vmcnt<NLOADS + EPI_STORES>(); else wait_vmcnt<NLOADS>(); }
+            else { if (sb) wait_vmcnt<EPI_STORES>(); else wait_vmcnt<0>(); }
+        }
         __syncthreads();
-        if (nkb > 1) {
+        if (nkb > NSTAGE - 1) {
             [&]<int... Q>(std::integer_sequence<int, Q...>) {
-                (issue_one(cp, 1, 1, std::integral_constant<int, Q>{}), ...);
+                (issue_one(cp, NSTAGE - 1, NSTAGE - 1, std::integral_constant<int, Q>{}), ...);
             }(std::make_integer_sequence<int, NL_LATE>{});
         }
 
@@ -409,48 +476,70 @@ void gemm_tr_kernel(const GemmArgs p) {
             read_b(breg[0], 0, lds);
         }
 
+        // All K blocks of the tile.  UB: the wave's n tiles [UB, NT) belong to the next b_scale block
+        // (UB = NT: none does).
+        auto run_blocks = [&](auto ub_tag) {
+        constexpr int UB = decltype(ub_tag)::value;
         // One K block (index j, in stage j&1).  The flags are compile-time so that the step sequence
         // is one straight-line block for the instruction scheduler.
-        auto k_block = [&](int j, auto has_next_tag, auto has_next2_tag) {
-            constexpr bool HAS_NEXT = decltype(has_next_tag)::value;      // block j+1 exists
-            constexpr bool HAS_NEXT2 = decltype(has_next2_tag)::value;    // block j+2 exists
-            const int cur_stage = j & 1;
+        // Block j lives in stage j % NSTAGE.  While it is multiplied, the rest of block j+NSTAGE-1 is
+        // copied into the stage that the barrier of block j-1 freed; behind the barrier of block j the
+        // first copies of block j+NSTAGE go into the stage just read.  With two stages a copy has one
+        // block's time to land, with three stages two.
+        auto k_block = [&](int j, auto h1_tag, auto h2_tag, auto h3_tag) {
+            constexpr bool HAS_NEXT = decltype(h1_tag)::value;                                              // block j+1 exists
+            constexpr bool HAS_EARLY = NSTAGE == 2 ? decltype(h1_tag)::value : decltype(h2_tag)::value;    // block j+NSTAGE-1 exists
+            constexpr bool HAS_LATE = NSTAGE == 2 ? decltype(h2_tag)::value : decltype(h3_tag)::value;     // block j+NSTAGE exists
+            const int cur_stage = NSTAGE == 2 ? (j & 1) : j % NSTAGE;
+            const int next_stage = cur_stage + 1 == NSTAGE ? 0 : cur_stage + 1;
+            const int early_stage = NSTAGE == 2 ? next_stage : (next_stage + 1 == NSTAGE ? 0 : next_stage + 1);
+            // what must have landed at the barrier is block j+1; with three stages the NLOADS copies of
+            // block j+2 were all issued after it and may stay in flight
+            auto wait_next_block = [&]() {
+                if constexpr (NSTAGE == 3 && HAS_EARLY) wait_vmcnt_lgkm0<NLOADS>();
+                else __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
+            };
             if (!wave_active) {
                 // none of this wave's rows is stored: it only does its share of the copies, in the
                 // same order and around the same single barrier as the waves that compute
-                if constexpr (HAS_NEXT) {
+                if constexpr (HAS_EARLY) {
                     [&]<int... Q>(std::integer_sequence<int, Q...>) {
-                        (issue_one(cp, cur_stage ^ 1, j + 1, std::integral_constant<int, NL_LATE + Q>{}), ...);
+                        (issue_one(cp, early_stage, j + NSTAGE - 1, std::integral_constant<int, NL_LATE + Q>{}), ...);
                     }(std::make_integer_sequence<int, NL_EARLY>{});
                 }
-                __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
+                wait_next_block();
                 __syncthreads();
-                if constexpr (HAS_NEXT2) {
+                if constexpr (HAS_LATE) {
                     [&]<int... Q>(std::integer_sequence<int, Q...>) {
-                        (issue_one(cp, cur_stage, j + 2, std::integral_constant<int, Q>{}), ...);
+                        (issue_one(cp, cur_stage, j + NSTAGE, std::integral_constant<int, Q>{}), ...);
                     }(std::make_integer_sequence<int, NL_LATE>{});
                 }
                 return;
             }
             const unsigned char* sbase = lds + cur_stage * C::STAGE_BYTES;
-            const unsigned char* snext = lds + (cur_stage ^ 1) * C::STAGE_BYTES;
-            float sc[C::MT];
+            const unsigned char* snext = lds + next_stage * C::STAGE_BYTES;
+            float sc[C::MT], sc1[C::MT];
             const float bsv = *(const float*)(sbase + bs_off);
+            const float bsv1 = UB < C::NT ? *(const float*)(sbase + bs_off + 4) : 0.f;
 #pragma unroll
-            for (int t = 0; t < C::MT; t++) sc[t] = *(const float*)(sbase + as_lane_off + t * 64) * bsv;
+            for (int t = 0; t < C::MT; t++) {
+                const float asv = *(const float*)(sbase + as_lane_off + t * 64);
+                sc[t] = asv * bsv;
+                sc1[t] = UB < C::NT ? asv * bsv1 : 0.f;
+            }
             v4f ring[RING];
             auto step = [&](auto s_tag) {
                 constexpr int s = decltype(s_tag)::value;
                 if constexpr (s < STEPS) {
                     constexpr int u = s / C::MT, t = s % C::MT;
-                    if constexpr (HAS_NEXT && s % DMA_EVERY == DMA_FIRST && s / DMA_EVERY < NL_EARLY)
-                        issue_one(cp, cur_stage ^ 1, j + 1, std::integral_constant<int, NL_LATE + s / DMA_EVERY>{});
+                    if constexpr (HAS_EARLY && s % DMA_EVERY == DMA_FIRST && s / DMA_EVERY < NL_EARLY)
+                        issue_one(cp, early_stage, j + NSTAGE - 1, std::integral_constant<int, NL_LATE + s / DMA_EVERY>{});
                     if constexpr (t == 0 && u + 1 < C::NT) read_b(breg[(u + 1) & 1], u + 1, sbase);
                     if constexpr (t == 0 && u == C::NT - 1) {
                         // All reads of this stage are issued.  Wait for them and for this wave's part
                         // of the next block, then meet the other waves: after the barrier the next
                         // block is complete in the other stage and this stage may be overwritten.
-                        __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
+                        wait_next_block();
                         __syncthreads();
                     }
                     const v4f z = {0.f, 0.f, 0.f, 0.f};
@@ -460,13 +549,13 @@ void gemm_tr_kernel(const GemmArgs p) {
                         read_a(areg[t], t, snext);
                         if constexpr (t == 0) read_b(breg[0], 0, snext);
                     }
-                    if constexpr (u == C::NT - 1 && HAS_NEXT2 && t < NL_LATE)
-                        issue_one(cp, cur_stage, j + 2, std::integral_constant<int, t>{});
+                    if constexpr (u == C::NT - 1 && HAS_LATE && t < NL_LATE)
+                        issue_one(cp, cur_stage, j + NSTAGE, std::integral_constant<int, t>{});
                 }
                 if constexpr (s >= LAG) {
                     constexpr int sp = s - LAG, u = sp / C::MT, t = sp % C::MT;
 #pragma unroll
-                    for (int r = 0; r < 4; r++) acc[t][u][r] = __builtin_fmaf(ring[sp % RING][r], sc[t], acc[t][u][r]);
+                    for (int r = 0; r < 4; r++) acc[t][u][r] = __builtin_fmaf(ring[sp % RING][r], u < UB ? sc[t] : sc1[t], acc[t][u][r]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             };
@@ -475,24 +564,45 @@ void gemm_tr_kernel(const GemmArgs p) {
             }(std::make_integer_sequence<int, STEPS + LAG>{});
         };
 
+        constexpr std::true_type T{};
+        constexpr std::false_type F{};
         int j = 0;
-        for (; j + 2 < nkb; j++) k_block(j, std::true_type{}, std::true_type{});
-        if (j + 1 < nkb) { k_block(j, std::true_type{}, std::false_type{}); j++; }
-        k_block(j, std::false_type{}, std::false_type{});
+        if constexpr (NSTAGE == 2) {
+            for (; j + 2 < nkb; j++) k_block(j, T, T, F);
+            if (j + 1 < nkb) { k_block(j, T, F, F); j++; }
+        } else {
+            for (; j + 3 < nkb; j++) k_block(j, T, T, T);
+            if (j + 2 < nkb) { k_block(j, T, T, F); j++; }
+            if (j + 1 < nkb) { k_block(j, T, F, F); j++; }
+        }
+        k_block(j, F, F, F);
+        };   // run_blocks
+        if constexpr (C::SPLIT_SCALES) {
+            // 96-column wave tiles of a 192-column tile start 0, 96, 64 or 160 columns into a block
+            if (ub == 2) run_blocks(std::integral_constant<int, 2>{});
+            else if (ub == 4) run_blocks(std::integral_constant<int, 4>{});
+            else run_blocks(std::integral_constant<int, C::NT>{});
+        } else {
+            run_blocks(std::integral_constant<int, C::NT>{});
+        }
     }
 
     else if (it > 0) {
         __syncthreads();                    // nothing to multiply: still let the previous tile's staging reads finish
     }
 
-    // ---- the next tile's first K block starts now: after the last barrier above no wave reads a
-    //      stage any more, and the output below is staged in stage 1 only ----
+    // ---- the next tile's first K blocks (all stages but the last) start now: after the last barrier
+    //      above no wave reads a stage any more, and the output below is staged in the last stage only ----
     Tile nxt = pick_tile(it + 1);
     CopyPlan ncp = cp;
     prefetched = false;
     if (nxt.valid) {
         ncp = copy_plan(nxt);
-        if (nxt.kb_end > nxt.kb_begin) { issue_all(ncp, 0, 0); prefetched = true; }
+        if (nxt.kb_end > nxt.kb_begin) {
+            issue_all(ncp, 0, 0);
+            if constexpr (NSTAGE == 3) { if (nxt.kb_end - nxt.kb_begin > 1) issue_all(ncp, 1, 1); }
+            prefetched = true;
+        }
     }
 
     // ---- epilogue (a wave without valid rows has nothing to store; no barrier in here) -----------
@@ -512,17 +622,21 @@ void gemm_tr_kernel(const GemmArgs p) {
         }
     } else {
         // bf16 through LDS so that the global stores are 16 bytes per lane and every store
-        // instruction writes whole rows of the wave tile (WNO*2 contiguous bytes each).  Stage 1 is
-        // free (after the barrier of the last K block no wave reads it and no copy into it is in
-        // flight); stage 0 already receives the next tile.  Each wave stages its tile in two halves of
+        // instruction writes whole rows of the wave tile (WNO*2 contiguous bytes each).  The last
+        // stage is free (after the barrier of the last K block no wave reads it and no copy into it is in
+        // flight); the stages before it already receive the next tile.  Each wave stages its tile in two halves of
         // WM/2 rows in its own region; 16-byte chunks are XOR-swizzled by row so that neither the
         // writes (16 rows per instruction) nor the 16-byte reads conflict.
         constexpr int WNO = EPI == 1 ? WN / 2 : WN;                   // output columns of the wave tile
         constexpr int ROW_CHUNKS = WNO * 2 / 16;                      // 16-byte chunks per tile row
         constexpr int ROWS_PER_SWEEP = 16 / ROW_CHUNKS > 0 ? 16 / ROW_CHUNKS : 1;
         constexpr int HALF_ROWS = WM / 2, HALF_MT = C::MT / 2;
-        static_assert(C::MT % 2 == 0 && C::NWAVES * HALF_ROWS * WNO * 2 <= C::STAGE_BYTES, "output staging must fit one stage");
-        unsigned char* region = lds + C::STAGE_BYTES + wave * (HALF_ROWS * WNO * 2);
+        // A row of 12 chunks is staged with one chunk of padding instead of the XOR swizzle: with 13
+        // chunks from row to row, 16 consecutive rows of one chunk column fall on 16 different bank groups.
+        constexpr bool ROW_POW2 = (ROW_CHUNKS & (ROW_CHUNKS - 1)) == 0;
+        constexpr int RSTRIDE = ROW_POW2 ? WNO * 2 : WNO * 2 + 16;    // bytes from row to row in the staging area
+        static_assert(C::MT % 2 == 0 && C::NWAVES * HALF_ROWS * RSTRIDE <= C::STAGE_BYTES, "output staging must fit one stage");
+        unsigned char* region = lds + (NSTAGE - 1) * C::STAGE_BYTES + wave * (HALF_ROWS * RSTRIDE);
         const int ldc = EPI == 1 ? p.n / 2 : p.n;
         // Stores go through buffer descriptors: an offset of 0xFFFFFFFF drops the lane's store, so the
         // instruction count does not depend on the data.  Each store gets a descriptor based at the first
@@ -532,42 +646,46 @@ void gemm_tr_kernel(const GemmArgs p) {
         // stores without a scalar offset).
         const int col0 = EPI == 1 ? n0 / 2 : n0;
         uint16_t* const c_tile = p.c + (size_t)m0 * ldc + col0;
-        static_assert(MODE == 1 || EPI_STORES == 2 * (HALF_ROWS * ROW_CHUNKS / 64), "store count used by the next tile's wait");
 #pragma unroll
         for (int half = 0; half < 2; half++) {
 #pragma unroll
             for (int th = 0; th < HALF_MT; th++) {
                 const int t = half * HALF_MT + th;
                 const int r = 16 * th + i16;
-                const int sw = (r / ROWS_PER_SWEEP) % ROW_CHUNKS;
+                const int sw = ROW_POW2 ? (r / ROWS_PER_SWEEP) % ROW_CHUNKS : 0;
 #pragma unroll
                 for (int u = 0; u < C::NT; u++) {
                     if (EPI == 1) {
                         // the lane's four columns are two (gate, up) pairs -> two outputs, 4 bytes
                         const uint32_t o = pack_bf16x2(silu_mul(acc[t][u][0], acc[t][u][1]), silu_mul(acc[t][u][2], acc[t][u][3]));
-                        *(uint32_t*)(region + r * (WNO * 2) + ((u ^ sw) << 4) + g * 4) = o;
+                        *(uint32_t*)(region + r * RSTRIDE + ((u ^ sw) << 4) + g * 4) = o;
                     } else {
                         v2i o;
                         o[0] = (int)pack_bf16x2(acc[t][u][0], acc[t][u][1]);
                         o[1] = (int)pack_bf16x2(acc[t][u][2], acc[t][u][3]);
                         const int chunk = 2 * u + (g >> 1);
-                        *(v2i*)(region + r * (WNO * 2) + ((chunk ^ sw) << 4) + (g & 1) * 8) = o;
+                        *(v2i*)(region + r * RSTRIDE + ((chunk ^ sw) << 4) + (g & 1) * 8) = o;
                     }
                 }
             }
-            constexpr int PASSES = HALF_ROWS * ROW_CHUNKS / 64, ROWS_PER_PASS = 64 / ROW_CHUNKS;
-            static_assert(HALF_ROWS * ROW_CHUNKS % 64 == 0 && 64 % ROW_CHUNKS == 0, "a half tile is a whole number of 16-byte sweeps");
+            // A pass = one 16-byte store per lane.  With 12 chunks per row a pass covers 4 rows with 48 lanes
+            // (the other 16 are switched off like out-of-range ones), so that, as in the power-of-two
+            // case, a lane keeps its row-in-pass and chunk over all passes.
+            constexpr int ROWS_PER_PASS = ROW_POW2 ? 64 / ROW_CHUNKS : 4, PASSES = HALF_ROWS / ROWS_PER_PASS;
+            static_assert(HALF_ROWS % ROWS_PER_PASS == 0 && ROWS_PER_PASS * ROW_CHUNKS <= 64, "a half tile is a whole number of passes");
+            static_assert(MODE == 1 || EPI_STORES == 2 * PASSES, "store count used by the next tile's wait");
             // lane -> (row inside the pass, chunk); everything else about a store's address is uniform
             // and sits in the descriptor, so the 16 stores need one address register, not 16
             const int lane_r = lane / ROW_CHUNKS, lane_chunk = lane % ROW_CHUNKS;
+            const bool lane_live = ROW_POW2 || lane_r < ROWS_PER_PASS;
             const int wave_row0 = wave_m * WM, wave_col0 = wave_n * WNO;              // inside the tile, output columns
-            const bool col_ok = col0 + wave_col0 + lane_chunk * 8 < ldc;
+            const bool col_ok = lane_live && col0 + wave_col0 + lane_chunk * 8 < ldc;
             const uint32_t lane_off = ((uint32_t)(wave_row0 + lane_r) * (uint32_t)ldc + (uint32_t)(wave_col0 + lane_chunk * 8)) * 2u;
 #pragma unroll
             for (int q = 0; q < PASSES; q++) {
-                const int r = q * ROWS_PER_PASS + lane_r;
-                const int sw = (r / ROWS_PER_SWEEP) % ROW_CHUNKS;
-                const v4i val = *(const v4i*)(region + r * (WNO * 2) + ((lane_chunk ^ sw) << 4));
+                const int r = q * ROWS_PER_PASS + (lane_live ? lane_r : 0);
+                const int sw = ROW_POW2 ? (r / ROWS_PER_SWEEP) % ROW_CHUNKS : 0;
+                const v4i val = *(const v4i*)(region + r * RSTRIDE + ((lane_chunk ^ sw) << 4));
                 const int pass_row0 = half * HALF_ROWS + q * ROWS_PER_PASS;            // compile-time
                 const int row = m0 + wave_row0 + pass_row0 + lane_r;
                 const bool ok = col_ok && row >= row_lo && row < row_hi;
@@ -883,10 +1001,10 @@ void gemm_generic_kernel(const GemmArgs p) {
 // ---------------------------------------------------------------------------------------------------
 // Launchers
 // ---------------------------------------------------------------------------------------------------
-template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0>
+template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0, int NSTAGE = 2>
 static hipError_t launch_tr(const GemmArgs& a, dim3 grid, hipStream_t stream) {
-    using C = TileCfg<BM, BN, WM, WN, MODE>;
-    auto kern = gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI>;
+    using C = TileCfg<BM, BN, WM, WN, MODE, NSTAGE>;
+    auto kern = gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI, NSTAGE>;
     static int raised[MAX_DEVICES];
     hipError_t e = raise_lds_limit((const void*)kern, C::LDS_BYTES, raised);
     if (e != hipSuccess) return e;
@@ -905,9 +1023,9 @@ static int device_cus() {
     return n;
 }
 
-template <int BM, int BN, int WM, int WN, bool WITH_EPI = false>
+template <int BM, int BN, int WM, int WN, bool WITH_EPI = false, int NSTAGE = 2>
 static hipError_t launch_shape(const GemmArgs& a, int mode, hipStream_t stream) {
-    using C = TileCfg<BM, BN, WM, WN, 0>;
+    using C = TileCfg<BM, BN, WM, WN, 0, NSTAGE>;
     // persistent workgroups: as many as fit the chip at once (LDS and thread limits), each walks
     // tiles  blockIdx.x, blockIdx.x + grid, ...
     const int by_lds = 163840 / C::LDS_BYTES, by_threads = 2048 / C::NTHREADS;
@@ -932,9 +1050,9 @@ static hipError_t launch_shape(const GemmArgs& a, int mode, hipStream_t stream) 
             return hipErrorInvalidValue;
         }
     }
-    if (mode == 2) return launch_tr<BM, BN, WM, WN, 2>(a, grid, stream);
-    if (mode == 1) return launch_tr<BM, BN, WM, WN, 1>(a, grid, stream);
-    return launch_tr<BM, BN, WM, WN, 0>(a, grid, stream);
+    if (mode == 2) return launch_tr<BM, BN, WM, WN, 2, 0, NSTAGE>(a, grid, stream);
+    if (mode == 1) return launch_tr<BM, BN, WM, WN, 1, 0, NSTAGE>(a, grid, stream);
+    return launch_tr<BM, BN, WM, WN, 0, 0, NSTAGE>(a, grid, stream);
 }
 
 template <int BN, int NSTAGE>
@@ -981,6 +1099,8 @@ hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t str
         case 6: return launch_skinny<144, 4>(a, mode, stream);
         case 7: return launch_skinny<256, 3>(a, mode, stream);
         case 8: return launch_skinny<288, 3>(a, mode, stream);
+        case 9: return launch_shape<256, 192, 64, 96>(a, mode, stream);
+        case 10: return launch_shape<256, 128, 64, 64, false, 3>(a, mode, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -1020,6 +1140,8 @@ int variant_lds_bytes(int variant) {
         case 6: return SkinnyCfg<144, 4>::LDS_BYTES;
         case 7: return SkinnyCfg<256, 3>::LDS_BYTES;
         case 8: return SkinnyCfg<288, 3>::LDS_BYTES;
+        case 9: return TileCfg<256, 192, 64, 96, 0>::LDS_BYTES;
+        case 10: return TileCfg<256, 128, 64, 64, 0, 3>::LDS_BYTES;
         default: return 0;
     }
 }

@@ -52,7 +52,9 @@ enum {
     FP8BS_VARIANT_SKINNY64x144 = 6, /* bandwidth-bound: 64(m) x 144(n) tile, 4-stage copy ring */
     FP8BS_VARIANT_SKINNY64x256 = 7, /* same, 256-wide tile (whole 128-byte lines), 3 stages      */
     FP8BS_VARIANT_SKINNY64x288 = 8, /* same, 288-wide tile, 3 stages                             */
-    FP8BS_VARIANT_COUNT = 9
+    FP8BS_VARIANT_T256x192 = 9,   /* 256(m) x 192(n) tile, 8 waves: fills more CUs when n/256 rounds up badly */
+    FP8BS_VARIANT_T256x128S3 = 10, /* 256 x 128 tile, three LDS stages (a copy has two K blocks' time to land) */
+    FP8BS_VARIANT_COUNT = 11
 };
 
 /* What fp8bs_plan() decides for a shape. Replaces the exact-(m,n,k) if-ladder of the reference

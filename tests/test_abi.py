@@ -40,11 +40,15 @@ def test_plan_shape_families(pkg):
     assert p.variant == q.variant != 1 and p.workspace_bytes == q.workspace_bytes + 1280   # 4*256 + 16*2 -> 1280
     assert pkg.plan(3, 190, 256).variant == 1
     p = pkg.plan(256, 512, 1024)                        # small: one of the sub-256 tiles, never the scalar kernel
-    assert p.variant in (3, 4, 5) and p.split_k >= 1 and p.split_k <= 8
+    assert p.variant in (3, 4, 10) and p.split_k >= 1 and p.split_k <= 8
     p = pkg.plan(1024, 512, 7168)                       # few tiles, long K: the planner splits K
-    assert p.variant in (3, 4, 5) and p.split_k > 1
+    assert p.variant in (3, 4, 10) and p.split_k > 1
     p = pkg.plan(6144, 4608, 7168)                      # large: the 256x256 tile, no split
     assert p.variant == 2 and p.split_k == 1
+    p = pkg.plan(4096, 2112, 7168)                      # 2112 = 11 x 192: 176 tiles of 256x192 instead of 144 of 256x256, 16 of them a quarter full
+    assert p.variant == 9 and (p.tile_m, p.tile_n) == (256, 192) and p.grid_x == 176 and p.lds_bytes == 2 * (128 * 448 + 1024 + 256)
+    p = pkg.plan(4096, 2048, 8192)                      # 256 tiles of 256x128, three stages
+    assert p.variant == 10 and (p.tile_m, p.tile_n) == (256, 128) and p.lds_bytes == 3 * (128 * 384 + 1024 + 256)
 
 
 def test_plan_rejects_bad_shapes(pkg):

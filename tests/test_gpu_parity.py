@@ -62,14 +62,14 @@ def test_config1_and_entry_point_contract(pkg, oracle, dev):
 
 def test_golden_fixture_bit_exact(pkg, golden_gemm, dev):
     cpu, expected, _ = golden_gemm
-    for variant in (0, 1, 3, 4, 6, 7, 8): # planner's choice, generic, 128x128 tile, 64x128 tile, the three ring kernels
+    for variant in (0, 1, 3, 4, 6, 7, 8, 9, 10): # planner's choice, generic, 128x128 tile, 64x128 tile, the three ring kernels, 256x192 tile, three-stage 256x128
         out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1 if variant else 0)
         assert torch.equal(out.cpu().view(torch.int16), expected.view(torch.int16)), "variant %d" % variant
     out = pkg.custom_kernel(_to(cpu, dev), variant=4, split_k=2)            # exact data: split-K is exact too
     assert torch.equal(out.cpu().view(torch.int16), expected.view(torch.int16))
 
 
-@pytest.mark.parametrize("variant,split_k", [(1, 1), (2, 1), (3, 1), (4, 1), (5, 1), (6, 1), (2, 2), (3, 3), (4, 4), (5, 8), (4, 7), (6, 2), (6, 8), (7, 1), (7, 2), (7, 3), (8, 1), (8, 4)])
+@pytest.mark.parametrize("variant,split_k", [(1, 1), (2, 1), (3, 1), (4, 1), (5, 1), (6, 1), (2, 2), (3, 3), (4, 4), (5, 8), (4, 7), (6, 2), (6, 8), (7, 1), (7, 2), (7, 3), (8, 1), (8, 4), (9, 1), (9, 2), (9, 8), (10, 1), (10, 2), (10, 3), (10, 4), (10, 8)])
 def test_every_variant_and_split_on_config1(pkg, oracle, dev, variant, split_k):
     cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0])
     out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=split_k)
@@ -91,13 +91,15 @@ def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
     if n % 8 == 0:
         assert pkg.plan(m, n, k).variant != 1                   # any m: the vector kernels, in two launches if m % 4 != 0
     if m % 4 == 0 and n % 8 == 0:
-        for variant in (2, 3, 4, 5, 6, 7, 8):
+        for variant in (2, 3, 4, 5, 6, 7, 8, 9, 10):
             out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1)
             _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d" % (m, n, k, variant))
 
 
 @pytest.mark.parametrize("m,n,k,variant", [(8192, 8192, 256, 2), (8188, 4104, 128, 0), (4096, 8192, 384, 5),
-                                           (8192, 4096, 256, 3), (4096, 4096, 256, 4)])
+                                           (8192, 4096, 256, 3), (4096, 4096, 256, 4),
+                                           (8192, 8256, 256, 9), (4100, 2112, 384, 9), (4096, 6336, 128, 9),
+                                           (8192, 8192, 128, 10), (8192, 4096, 256, 10), (4100, 8200, 384, 10), (4096, 4096, 512, 10)])
 def test_many_tiles_per_workgroup_against_the_scalar_kernel(pkg, oracle, dev, m, n, k, variant):
     """Short K and a large output: every persistent workgroup walks many tiles, so the hand-over between
     tiles (next tile's first block issued ahead of the output stores, counted wait) carries the result.
