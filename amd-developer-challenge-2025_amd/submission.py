@@ -153,8 +153,9 @@ def custom_kernel(data, variant: int = 0, split_k: int = 0):
     return c
 
 
-def grouped_kernel(data):
+def grouped_kernel(data, variant: int = 0):
     """Grouped (MoE expert) variant: ``data = (a, b, a_scale, b_scale, row_offsets, c)``.
+    ``variant`` forces a tile (FP8BS_VARIANT_*) for testing; 0 lets the library choose.
 
     Row-offset convention of 2-amd-moe/3-amd-fp8-moe-hip-myhgemm.py:142-148, :328-336 with the
     total appended: ``row_offsets`` is int32 [E+1] on the GPU, expert e owns rows
@@ -176,7 +177,7 @@ def grouped_kernel(data):
     lib = _lib.load()
     with torch.cuda.device(a.device):
         stream = torch.cuda.current_stream().cuda_stream
-        st = lib.fp8bs_gemm_grouped(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
-                                    c.data_ptr(), row_offsets.data_ptr(), num_experts, rows, n, k, stream)
+        st = lib.fp8bs_gemm_grouped_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
+                                       c.data_ptr(), row_offsets.data_ptr(), num_experts, rows, n, k, variant, stream)
     _lib.check(st)
     return c

@@ -116,6 +116,13 @@ int fp8bs_gemm_grouped(const void* a, const void* b, const float* a_scale, const
                        void* c, const int32_t* row_offsets, int num_experts, int total_rows,
                        int n, int k, void* stream);
 
+/* Same with the tile forced: one of the FP8BS_VARIANT_T* tiles or FP8BS_VARIANT_GENERIC (the streaming
+ * variants have no grouped mode: FP8BS_ERR_BAD_VARIANT).  FP8BS_VARIANT_AUTO reproduces
+ * fp8bs_gemm_grouped (the 256x256 tile, or the scalar kernel for shapes and pointers off the 16-byte grid). */
+int fp8bs_gemm_grouped_ex(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                          void* c, const int32_t* row_offsets, int num_experts, int total_rows,
+                          int n, int k, int variant, void* stream);
+
 /* ---- Quantisers (the step in front of the GEMM) -------------------------------------------------
  * The reference has no counterpart: its operands arrive already quantised from the harness
  * (1-amd-fp8-mm/0-amd-fp8-mm-new-begins.py:66-77).  These produce exactly those operands, in the

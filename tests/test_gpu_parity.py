@@ -310,6 +310,33 @@ def test_grouped_every_element_against_the_scalar_kernel(pkg, dev):
     assert int(bad.sum()) == 0, "%d elements differ, first at %s" % (int(bad.sum()), bad.nonzero()[0].tolist())
 
 
+@pytest.mark.parametrize("variant", [2, 3, 4, 5, 9, 10])
+@pytest.mark.parametrize("tokens,experts,topk,n,k", [(96, 8, 2, 448, 384), (1024, 32, 8, 2112, 256), (40, 16, 1, 256, 128)])
+def test_grouped_with_every_tile_against_the_scalar_kernel(pkg, dev, variant, tokens, experts, topk, n, k):
+    """Every tile shape in grouped mode: experts of a few rows, empty experts (40 tokens over 16 experts), expert boundaries inside a
+    tile and inside a 16-row group, column tails.  Every element against the scalar kernel."""
+    cfg = pkg.inputs.CONFIGS[4]
+    data = list(_to(pkg.inputs.make_grouped(cfg, tokens=tokens, experts=experts, topk=topk, n=n, k=k), dev))
+    rows = data[0].shape[0]
+    if rows % 4:
+        pytest.skip("the vector kernels need a multiple of four rows")
+    ref = pkg.grouped_kernel(tuple(data[:5]) + (torch.full_like(data[5], float("nan")),), variant=1).float()
+    out = pkg.grouped_kernel(tuple(data[:5]) + (torch.full_like(data[5], float("nan")),), variant=variant).float()
+    auto = pkg.grouped_kernel(tuple(data[:5]) + (torch.full_like(data[5], float("nan")),)).float()
+    assert not bool(ref.isnan().any())
+    for name, got in (("variant %d" % variant, out), ("library's choice", auto)):
+        bad = ~((got - ref).abs() <= ATOL + RTOL * ref.abs())
+        assert int(bad.sum()) == 0, "%s: %d elements differ, first at %s" % (name, int(bad.sum()), bad.nonzero()[0].tolist())
+
+
+def test_grouped_refuses_the_streaming_variants(pkg, dev):
+    cfg = pkg.inputs.CONFIGS[4]
+    data = _to(pkg.inputs.make_grouped(cfg, tokens=64, experts=4, topk=2, n=256, k=128), dev)
+    for variant in (6, 7, 8, 99):
+        with pytest.raises(Exception):
+            pkg.grouped_kernel(data, variant=variant)
+
+
 def test_special_codes(pkg, oracle, dev):
     """-0, the largest codes (+-448), the smallest subnormals and NaN codes: a NaN in a row of A or B
     poisons exactly the outputs that row takes part in, everything else stays within the bar."""
