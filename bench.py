@@ -252,6 +252,21 @@ def main():
         fl = 2.0 * rows * cfg5.n * cfg5.k
         per_config["ffn_gate_up_silu_32768x4096x7168"] = {"us": round(us, 2), "us_min": round(us_min, 2), "tflops": round(fl / us * 1e-6, 1),
                                                           "bound": "mfma", "frac": round(fl / us * 1e-6 / PEAK_FP8_TFLOPS, 4)}
+        # a decode step through the same weights: 32 tokens x 8 experts = 256 rows, 8 per expert on
+        # average; the call streams every expert's gate/up weights once (940 MB, more than the 256 MB cache)
+        dec_rows = 32 * cfg5.topk
+        gdec = torch.Generator(device=dev).manual_seed(11)
+        counts = torch.bincount(torch.randint(0, cfg5.experts, (dec_rows,), generator=gdec, device=dev), minlength=cfg5.experts)
+        ro_dec = torch.zeros(cfg5.experts + 1, dtype=torch.int32, device=dev)
+        ro_dec[1:] = torch.cumsum(counts, 0).to(torch.int32)
+        a_dec, as_dec = quant.quantize_a(torch.randn(dec_rows, cfg5.k, generator=gdec, device=dev))
+        c_dec = torch.empty(dec_rows, cfg5.n, dtype=torch.bfloat16, device=dev)
+        us, us_min = time_calls(lambda i: pkg.grouped_kernel((a_dec, b5, as_dec, bs5, ro_dec, c_dec)), max(args.steps // 5, 5), 3)
+        by = cfg5.experts * cfg5.n * cfg5.k + 4 * cfg5.experts * (cfg5.n // 128) * (cfg5.k // 128) + dec_rows * cfg5.k + 4 * dec_rows * (cfg5.k // 128) + 2 * dec_rows * cfg5.n
+        per_config["grouped_decode_256rows_32x4096x7168"] = {"us": round(us, 2), "us_min": round(us_min, 2), "gbs": round(by / us * 1e-3, 1), "bytes": by,
+                                                            "bound": "hbm", "frac": round(by / us * 1e-3 / PEAK_HBM_GBS, 4),
+                                                            "note": "grouped GEMM with ~8 rows per expert: bound by streaming the experts' weights"}
+        a_dec = as_dec = c_dec = ro_dec = None
         d5 = a5 = b5 = as5 = bs5 = None
         torch.cuda.empty_cache()
         di = cfg5.n // 2
