@@ -67,8 +67,9 @@ uint64_t pad4_bytes(int k) { return (((uint64_t)k * 4u + (uint64_t)(k / KBLK) * 
 // aligned.
 bool vector_shape(int m, int n) { return (m % 4) == 0 && (n % 8) == 0; }
 
-// Shape-family rule.  m not a multiple of 4 or n not a multiple of 8 -> generic kernel.  m > 128 -> the tiled MFMA kernel whose tile shape finishes soonest under a
-// small cost model.  m <= 128 -> the streaming kernel with the K split that fills the CUs.
+// Shape-family rule.  n not a multiple of 8 -> generic kernel; m not a multiple of 4 -> two launches.  Then
+// the tiled MFMA kernel whose tile shape and K split finish soonest under a small cost model, except for
+// a few rows against a very large B: the streaming kernel with the K split that fills the CUs.
 void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     if (num_cus <= 0) num_cus = 256;
     if (!vector_shape(m, n)) {
@@ -94,8 +95,14 @@ void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
         return;
     }
     int kbt = k / KBLK;
-    if (m > 128) {
-        // Compute-bound family: the tile shape and K split that finish soonest under a cost model in
+    // The streaming kernel is kept for what it was built for: at most 64 rows against a B too large for the
+    // caches (configuration 4: 132 MB).  Measured over m = 32 .. 128, n = 512 .. 18432, k = 2048 / 7168 the
+    // tiled kernels with a K split are level with it there (38 us either way on configuration 4) and ahead
+    // everywhere else: by 3-10 % on smaller B, by 25-30 % from 65 rows on, where the streaming kernel needs a
+    // second row of tiles and reads B twice.
+    const bool streaming = m <= 64 && (double)n * (double)k >= 96.0e6;
+    if (!streaming) {
+        // The tile shape and K split that finish soonest under a cost model in
         // microseconds.  Per variant and number r of workgroups resident on a CU, measured on MI355X
         // (K = 1024 and 8192 on shapes of exactly r workgroups per CU): the time in which all r advance
         // one K block, and the fixed time of a round (prologue, output, drain).  Workgroups are dealt in
@@ -134,7 +141,7 @@ void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
         return;
     }
     {
-        // Bandwidth-bound family (m <= 128): stream B once with the 64x144 ring kernel.  Pick the K split that
+        // Bandwidth-bound family: stream B once with the 64x144 ring kernel.  Pick the K split that
         // minimises (rounds over the CUs) x (K blocks per workgroup) x (bytes of B per workgroup and
         // K block) plus the fp32 partial planes the split writes and reads back.
         long tiles = cdiv(m, 64) * cdiv(n, 144);
