@@ -59,8 +59,11 @@ void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out)
     out->workspace_bytes = split_k > 1 ? (uint64_t)split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
 }
 
-// Bytes at the head of the workspace for the four-row copies of a and a_scale (m < 4).
-uint64_t pad4_bytes(int k) { return (((uint64_t)k * 4u + (uint64_t)(k / KBLK) * 16u) + 255u) & ~(uint64_t)255u; }
+// m not a multiple of four and at most this many rows: a and a_scale are copied into matrices of mp = m
+// rounded up to four rows at the head of the workspace (k * mp bytes: small next to one more pass over b,
+// which is what the two-launch scheme for larger m costs).
+constexpr int PAD_MAX_ROWS = 1024;
+uint64_t pad_bytes(int k, int mp) { return (((uint64_t)k * (uint64_t)mp + (uint64_t)(k / KBLK) * (uint64_t)mp * 4u) + 255u) & ~(uint64_t)255u; }
 
 // What the vector kernels need of a shape: rows of a (m bytes) that keep the 4-byte loads of a copy
 // aligned and inside the buffer's per-dword range check, rows of c (n bf16) that keep 16-byte stores
@@ -70,25 +73,27 @@ bool vector_shape(int m, int n) { return (m % 4) == 0 && (n % 8) == 0; }
 // Shape-family rule.  n not a multiple of 8 -> generic kernel; m not a multiple of 4 -> two launches.  Then
 // the tiled MFMA kernel whose tile shape and K split finish soonest under a small cost model, except for
 // a few rows against a very large B: the streaming kernel with the K split that fills the CUs.
-void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
+// m_all: rows of the whole call when m is only its first launch (m_all - m < 4 rows follow in a second one)
+void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out, int m_all = 0) {
     if (num_cus <= 0) num_cus = 256;
     if (!vector_shape(m, n)) {
-        // m not a multiple of 4: the planned kernel takes the first m - m % 4 rows (reading a with its
-        // true row length) and a second launch of the streaming kernel the last four rows (a window that
-        // ends exactly at the end of every k row, so the last dword of a is never cut by the buffer's
-        // range check).  The plan describes the first launch; the workspace covers both.
-        if ((n % 8) == 0 && (m & ~3) > 0) {
-            fp8bs_plan_t tail{};
-            choose(m & ~3, n, k, num_cus, out);
-            choose(4, n, k, num_cus, &tail);
-            if (tail.workspace_bytes > out->workspace_bytes) out->workspace_bytes = tail.workspace_bytes;
+        // m not a multiple of 4, up to PAD_MAX_ROWS rows: the operands are copied into matrices of
+        // mp = m rounded up to four rows at the head of the workspace and the planned kernel runs on those
+        if ((n % 8) == 0 && m <= PAD_MAX_ROWS) {
+            const int mp = (m + 3) & ~3;
+            choose(mp, n, k, num_cus, out);
+            out->workspace_bytes += pad_bytes(k, mp);
             return;
         }
-        // one to three rows (a few tokens of a decode step): the operands are copied into four-row
-        // matrices at the head of the workspace and the streaming kernel runs on those
-        if ((n % 8) == 0 && m < 4) {
-            choose(4, n, k, num_cus, out);
-            out->workspace_bytes += pad4_bytes(k);
+        // more rows: the planned kernel takes the first m - m % 4 rows (reading a with its true row
+        // length) and a second launch the last four rows (a window that ends exactly at the end of every
+        // k row, so the last dword of a is never cut by the buffer's range check).  The plan describes the
+        // first launch; the workspace covers both.
+        if ((n % 8) == 0 && (m & ~3) > 0) {
+            fp8bs_plan_t tail{};
+            choose(m & ~3, n, k, num_cus, out, m);
+            choose(4, n, k, num_cus, &tail);
+            if (tail.workspace_bytes > out->workspace_bytes) out->workspace_bytes = tail.workspace_bytes;
             return;
         }
         fill_plan(m, n, k, FP8BS_VARIANT_GENERIC, 1, out);
@@ -100,7 +105,7 @@ void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     // tiled kernels with a K split are level with it there (38 us either way on configuration 4) and ahead
     // everywhere else: by 3-10 % on smaller B, by 25-30 % from 65 rows on, where the streaming kernel needs a
     // second row of tiles and reads B twice.
-    const bool streaming = m <= 64 && (double)n * (double)k >= 96.0e6;
+    const bool streaming = (m_all > m ? m_all : m) <= 64 && (double)n * (double)k >= 96.0e6;
     if (!streaming) {
         // The tile shape and K split that finish soonest under a cost model in
         // microseconds.  Per variant and number r of workgroups resident on a CU, measured on MI355X
@@ -221,27 +226,28 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
         variant = FP8BS_VARIANT_GENERIC;
     }
     int m_main = m;                                    // rows the planned kernel computes
-    if (variant == FP8BS_VARIANT_AUTO && split_k == 0 && m < 4 && (n % 8) == 0 && k > 0) {
-        // one to three rows: four-row copies of a / a_scale at the head of the workspace, then the
-        // streaming kernel; without enough workspace the generic kernel below does it
-        choose(4, n, k, 0, &plan);
-        const uint64_t pad = pad4_bytes(k);
+    if (variant == FP8BS_VARIANT_AUTO && split_k == 0 && (m % 4) != 0 && m <= PAD_MAX_ROWS && (n % 8) == 0 && k > 0) {
+        // padded copies of a / a_scale at the head of the workspace, then the kernel planned for the padded
+        // row count; without enough workspace the two-launch scheme below (m >= 4) or the generic kernel
+        const int mp = (m + 3) & ~3;
+        choose(mp, n, k, 0, &plan);
+        const uint64_t pad = pad_bytes(k, mp);
         const uint64_t planes = plan.split_k > 1 ? (uint64_t)plan.split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
         if (ws && ws_bytes >= pad + planes) {
-            uint8_t* a4 = (uint8_t*)ws;
-            float* as4 = (float*)(a4 + (size_t)k * 4);
-            if (fp8bs::launch_pad_rows4((const uint8_t*)a, a_scale, a4, as4, m, k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
+            uint8_t* ap = (uint8_t*)ws;
+            float* asp = (float*)(ap + (size_t)k * mp);
+            if (fp8bs::launch_pad_rows((const uint8_t*)a, a_scale, ap, asp, m, mp, k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
             fp8bs::GemmArgs g{};
-            g.a = a4; g.b = (const uint8_t*)b; g.as = as4; g.bs = b_scale;
+            g.a = ap; g.b = (const uint8_t*)b; g.as = asp; g.bs = b_scale;
             g.c = (uint16_t*)c; g.ws = (float*)((uint8_t*)ws + pad); g.row_offsets = nullptr;
-            g.m = m; g.n = n; g.k = k; g.lda = 4; g.nb = (n + 127) / 128;
+            g.m = m; g.n = n; g.k = k; g.lda = mp; g.nb = (n + 127) / 128;
             g.split_k = plan.split_k; g.kb_per_split = (int)cdiv(k / KBLK, plan.split_k); g.band_h = 4;
             const int mode = plan.split_k > 1 ? 1 : 0;
             if (fp8bs::launch_gemm(plan.variant, mode, g, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
             if (mode == 1 && fp8bs::launch_splitk_reduce(g.ws, g.c, (size_t)m * n, plan.split_k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
             return FP8BS_OK;
         }
-        variant = FP8BS_VARIANT_GENERIC;
+        if (m < 4) variant = FP8BS_VARIANT_GENERIC;
     }
     if (variant == FP8BS_VARIANT_AUTO) {
         choose(m, n, k, 0, &plan);

@@ -1105,22 +1105,31 @@ hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t str
     }
 }
 
-// Fewer than four rows of a (one to three tokens): copy a and a_scale into four-row matrices (rows beyond
-// m are zero).  With four bytes per k row every load of the vector kernels stays on a dword of its own.
+// A number of rows that is not a multiple of four (a few tokens of a decode step, an odd batch): copy a
+// and a_scale into matrices of mp = m rounded up to four rows (the added rows are zero).  With k rows of
+// mp bytes every 4-byte load of the vector kernels stays on a dword of its own and inside the buffer.
 __global__ __launch_bounds__(256)
-void pad_rows4_kernel(const uint8_t* __restrict__ a, const float* __restrict__ as, uint8_t* __restrict__ a4, float* __restrict__ as4, int m, int k) {
-    const int kk = blockIdx.x * 256 + threadIdx.x;
-    if (kk < k) {
+void pad_rows_kernel(const uint8_t* __restrict__ a, const float* __restrict__ as, uint8_t* __restrict__ ap, float* __restrict__ asp, int m, int mp, int k) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const int groups = mp / 4;
+    if (idx < (size_t)k * groups) {
+        const size_t kk = idx / groups;
+        const int r0 = 4 * (int)(idx % groups);
         uint32_t w = 0;
-        for (int i = 0; i < m; i++) w |= (uint32_t)a[(size_t)kk * m + i] << (8 * i);
-        *(uint32_t*)(a4 + 4 * (size_t)kk) = w;
+        for (int i = 0; i < 4; i++)
+            if (r0 + i < m) w |= (uint32_t)a[kk * m + r0 + i] << (8 * i);
+        *(uint32_t*)(ap + 4 * idx) = w;
     }
-    if (kk < k / KBLK)
-        for (int i = 0; i < 4; i++) as4[4 * (size_t)kk + i] = i < m ? as[(size_t)kk * m + i] : 0.f;
+    if (idx < (size_t)(k / KBLK) * mp) {
+        const size_t kb = idx / mp;
+        const int r = (int)(idx % mp);
+        asp[idx] = r < m ? as[kb * m + r] : 0.f;
+    }
 }
 
-hipError_t launch_pad_rows4(const uint8_t* a, const float* as, uint8_t* a4, float* as4, int m, int k, hipStream_t stream) {
-    hipLaunchKernelGGL(pad_rows4_kernel, dim3((unsigned)((k + 255) / 256)), dim3(256), 0, stream, a, as, a4, as4, m, k);
+hipError_t launch_pad_rows(const uint8_t* a, const float* as, uint8_t* ap, float* asp, int m, int mp, int k, hipStream_t stream) {
+    const size_t threads = (size_t)k * (mp / 4);                  // more than the (k/128)*mp scale entries
+    hipLaunchKernelGGL(pad_rows_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, a, as, ap, asp, m, mp, k);
     return hipGetLastError();
 }
 

@@ -89,9 +89,10 @@ size_t fp8bs_workspace_bytes(int m, int n, int k);
  * 1-amd-fp8-mm/amd-fp8-mm-submission.py:514-579. Inputs are never modified (the reference's
  * pre-transpose branch, :570-571, overwrites a and b; this one does not).
  * Alignment: the fast kernels need n a multiple of 8 and a, b, c, ws on 16-byte boundaries (with m not a
- * multiple of 4 they take the first m - m % 4 rows and a second launch the last four rows; with m < 4
- * a and a_scale are first copied into four-row matrices at the head of the workspace - without one, the
- * generic kernel runs);
+ * multiple of 4: up to 1024 rows, a and a_scale are first copied into matrices of m rounded up to four
+ * rows at the head of the workspace; above that, or without enough workspace, the fast kernel takes the
+ * first m - m % 4 rows and a second launch the last four rows; m < 4 without a workspace runs on the
+ * generic kernel);
  * other shapes or pointers run on the element-wise generic kernel (correct, slow).  a_scale and
  * b_scale must be 4-byte aligned, c 2-byte aligned (FP8BS_ERR_BAD_SHAPE otherwise). */
 int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,

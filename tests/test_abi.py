@@ -34,8 +34,10 @@ def test_plan_shape_families(pkg):
     assert p.workspace_bytes == p.split_k * 64 * 18432 * 4 == pkg.workspace_bytes(64, 18432, 7168)
     p = pkg.plan(130, 190, 256)                         # n not a multiple of 8 -> generic kernel
     assert p.variant == 1 and p.split_k == 1
-    p, q = pkg.plan(130, 192, 256), pkg.plan(128, 192, 256)   # m % 4 != 0: the plan of the first 128 rows
-    assert p.variant == q.variant != 1 and p.split_k == q.split_k and p.workspace_bytes == q.workspace_bytes
+    p, q = pkg.plan(130, 192, 256), pkg.plan(132, 192, 256)   # m % 4 != 0, few rows: the plan of 132 rows on padded copies of a / a_scale
+    assert p.variant == q.variant != 1 and p.split_k == q.split_k and p.workspace_bytes == q.workspace_bytes + 35072   # 256*132 + 2*132*4 -> 35072
+    p, q = pkg.plan(4095, 512, 256), pkg.plan(4092, 512, 256) # many rows: the plan of the first 4092 rows, the last four in a second launch
+    assert p.variant == q.variant != 1 and p.split_k == q.split_k and p.workspace_bytes >= q.workspace_bytes
     p, q = pkg.plan(3, 192, 256), pkg.plan(4, 192, 256)       # 1..3 rows: four-row copies in the workspace
     assert p.variant == q.variant != 1 and p.workspace_bytes == q.workspace_bytes + 1280   # 4*256 + 16*2 -> 1280
     assert pkg.plan(3, 190, 256).variant == 1
@@ -49,6 +51,21 @@ def test_plan_shape_families(pkg):
     assert p.variant == 9 and (p.tile_m, p.tile_n) == (256, 192) and p.grid_x == 176 and p.lds_bytes == 2 * (128 * 448 + 1024 + 256)
     p = pkg.plan(4096, 2048, 8192)                      # 256 tiles of 256x128, three stages
     assert p.variant == 10 and (p.tile_m, p.tile_n) == (256, 128) and p.lds_bytes == 3 * (128 * 384 + 1024 + 256)
+
+
+def test_plan_streaming_kernel_only_for_few_rows_against_a_large_b(pkg):
+    """The streaming kernel is planned for at most 64 rows and a B of 96 MB or more; everything else goes
+    through the tiled kernels' cost model (more rows would make the streaming kernel copy B twice)."""
+    for m, n, k, streaming in [(64, 18432, 7168, True), (16, 18432, 7168, True), (4, 18432, 7168, True),
+                               (65, 18432, 7168, False), (128, 18432, 7168, False), (64, 7168, 7168, False),
+                               (64, 18432, 2048, False), (32, 512, 2048, False)]:
+        p = pkg.plan(m, n, k)
+        assert (p.variant in (6, 7, 8)) == streaming, (m, n, k, p.variant)
+        assert p.variant != 1
+        if m % 4 == 0:
+            assert p.workspace_bytes == (p.split_k * m * n * 4 if p.split_k > 1 else 0)
+    # one to three rows take the plan of four rows plus the padded copies
+    assert pkg.plan(1, 18432, 7168).variant == pkg.plan(4, 18432, 7168).variant == 6
 
 
 def test_plan_rejects_bad_shapes(pkg):

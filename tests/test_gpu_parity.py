@@ -80,7 +80,8 @@ def test_every_variant_and_split_on_config1(pkg, oracle, dev, variant, split_k):
                                    (64, 1024, 1024), (512, 144, 1280), (130, 192, 256), (1, 7, 128), (33, 129, 384),
                                    (132, 200, 256), (20, 24, 128), (516, 264, 384), (268, 2104, 256),
                                    (4095, 512, 256), (1021, 264, 384), (131, 1024, 512), (61, 2048, 1024), (5, 16, 128),
-                                   (1, 2048, 1024), (2, 264, 384), (3, 18432, 512)])
+                                   (1, 2048, 1024), (2, 264, 384), (3, 18432, 512), (5, 18432, 512), (1030, 264, 256), (2050, 136, 384),
+                                   (1023, 8, 128), (67, 2112, 640)])
 def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
     """N tails (2112 = 16*128 + 64), tiles larger than the matrix, rows and columns that end inside a
     16-byte chunk (m % 4 == 0, n % 8 == 0: still the vector kernels), shapes only the generic kernel takes."""
