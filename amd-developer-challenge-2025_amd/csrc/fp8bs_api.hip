@@ -59,106 +59,96 @@ void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out)
     out->workspace_bytes = split_k > 1 ? (uint64_t)split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
 }
 
-// m not a multiple of four and at most this many rows: a and a_scale are copied into matrices of mp = m
-// rounded up to four rows at the head of the workspace (k * mp bytes: small next to one more pass over b,
-// which is what the two-launch scheme for larger m costs).
-constexpr int PAD_MAX_ROWS = 1024;
+// The streaming kernels copy a in dwords that must not cross the end of its buffer: they need m % 4 == 0.
+// For other m, a and a_scale are first copied into matrices of mp = m rounded up to four rows at the head
+// of the workspace (k * mp bytes: the streaming kernels only ever see a few rows).
 uint64_t pad_bytes(int k, int mp) { return (((uint64_t)k * (uint64_t)mp + (uint64_t)(k / KBLK) * (uint64_t)mp * 4u) + 255u) & ~(uint64_t)255u; }
 
-// What the vector kernels need of a shape: rows of a (m bytes) that keep the 4-byte loads of a copy
-// aligned and inside the buffer's per-dword range check, rows of c (n bf16) that keep 16-byte stores
-// aligned.
-bool vector_shape(int m, int n) { return (m % 4) == 0 && (n % 8) == 0; }
+// What the vector kernels need of a shape: rows of c (n bf16) that keep 16-byte stores aligned.  The
+// tiled kernels take any m (they repair the last bytes of a themselves), the streaming kernels m % 4 == 0.
+bool vector_shape(int n) { return (n % 8) == 0; }
 
-// Shape-family rule.  n not a multiple of 8 -> generic kernel; m not a multiple of 4 -> two launches.  Then
-// the tiled MFMA kernel whose tile shape and K split finish soonest under a small cost model, except for
-// a few rows against a very large B: the streaming kernel with the K split that fills the CUs.
-// m_all: rows of the whole call when m is only its first launch (m_all - m < 4 rows follow in a second one)
-void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out, int m_all = 0) {
+// The streaming kernel is kept for what it was built for: at most 64 rows against a B too large for the
+// caches (configuration 4: 132 MB).  Measured over m = 32 .. 128, n = 512 .. 18432, k = 2048 / 7168 the
+// tiled kernels with a K split are level with it there (38 us either way on configuration 4) and ahead
+// everywhere else: by 3-10 % on smaller B, by 25-30 % from 65 rows on, where the streaming kernel needs a
+// second row of tiles and reads B twice.
+bool streaming_shape(int m, int n, int k) { return m <= 64 && (double)n * (double)k >= 96.0e6; }
+
+// The tile shape and K split of the tiled MFMA kernel that finish soonest (any m).
+void choose_tiled(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     if (num_cus <= 0) num_cus = 256;
-    if (!vector_shape(m, n)) {
-        // m not a multiple of 4, up to PAD_MAX_ROWS rows: the operands are copied into matrices of
-        // mp = m rounded up to four rows at the head of the workspace and the planned kernel runs on those
-        if ((n % 8) == 0 && m <= PAD_MAX_ROWS) {
-            const int mp = (m + 3) & ~3;
-            choose(mp, n, k, num_cus, out);
-            out->workspace_bytes += pad_bytes(k, mp);
-            return;
-        }
-        // more rows: the planned kernel takes the first m - m % 4 rows (reading a with its true row
-        // length) and a second launch the last four rows (a window that ends exactly at the end of every
-        // k row, so the last dword of a is never cut by the buffer's range check).  The plan describes the
-        // first launch; the workspace covers both.
-        if ((n % 8) == 0 && (m & ~3) > 0) {
-            fp8bs_plan_t tail{};
-            choose(m & ~3, n, k, num_cus, out, m);
-            choose(4, n, k, num_cus, &tail);
-            if (tail.workspace_bytes > out->workspace_bytes) out->workspace_bytes = tail.workspace_bytes;
-            return;
-        }
-        fill_plan(m, n, k, FP8BS_VARIANT_GENERIC, 1, out);
-        return;
-    }
     int kbt = k / KBLK;
-    // The streaming kernel is kept for what it was built for: at most 64 rows against a B too large for the
-    // caches (configuration 4: 132 MB).  Measured over m = 32 .. 128, n = 512 .. 18432, k = 2048 / 7168 the
-    // tiled kernels with a K split are level with it there (38 us either way on configuration 4) and ahead
-    // everywhere else: by 3-10 % on smaller B, by 25-30 % from 65 rows on, where the streaming kernel needs a
-    // second row of tiles and reads B twice.
-    const bool streaming = (m_all > m ? m_all : m) <= 64 && (double)n * (double)k >= 96.0e6;
-    if (!streaming) {
-        // The tile shape and K split that finish soonest under a cost model in
-        // microseconds.  Per variant and number r of workgroups resident on a CU, measured on MI355X
-        // (K = 1024 and 8192 on shapes of exactly r workgroups per CU): the time in which all r advance
-        // one K block, and the fixed time of a round (prologue, output, drain).  Workgroups are dealt in
-        // rounds of (CUs x the most that fit a CU); a last partial round runs with fewer per CU.  A K
-        // split adds the fp32 partial planes (written and read back, mostly through the 256 MB cache) and the
-        // reduce launch.
-        struct Cand { int variant; int rmax; double t_block[3], t_fixed[3]; };
-        const Cand cands[5] = {
-            {FP8BS_VARIANT_T256x256, 1, {1.87, 0, 0}, {6.8, 0, 0}},
-            {FP8BS_VARIANT_T256x192, 1, {1.45, 0, 0}, {6.0, 0, 0}},
-            {FP8BS_VARIANT_T256x128S3, 1, {1.18, 0, 0}, {4.2, 0, 0}},
-            {FP8BS_VARIANT_T128x128, 2, {0.89, 1.34, 0}, {3.1, 4.8, 0}},
-            {FP8BS_VARIANT_T64x128, 3, {0.70, 1.04, 1.39}, {1.9, 2.3, 3.6}},
-        };
-        const int splits[6] = {1, 2, 3, 4, 6, 8};
-        int best_variant = 0, best_split = 1; double best_cost = 0;
-        for (const Cand& c : cands) {
-            VariantInfo vi{};
-            variant_info(c.variant, &vi);
-            const long tiles = cdiv(m, vi.bm) * cdiv(n, vi.bn);
-            for (int s : splits) {
-                if (s > 1 && kbt / s < 4) continue;                  // keep at least 4 K blocks per workgroup
-                const long wgs = tiles * s, per_round = (long)num_cus * c.rmax;
-                const long full = wgs / per_round, rem = wgs % per_round;
-                const double kb = (double)cdiv(kbt, s);
-                double cost = (double)full * (c.t_fixed[c.rmax - 1] + kb * c.t_block[c.rmax - 1]);
-                if (rem) {
-                    const long r = cdiv(rem, num_cus);
-                    cost += c.t_fixed[r - 1] + kb * c.t_block[r - 1];
-                }
-                if (s > 1) cost += 2.0 + 8.0 * s * (double)m * (double)n / 8.0e6;
-                if (best_variant == 0 || cost < best_cost) { best_variant = c.variant; best_split = s; best_cost = cost; }
+    // The tile shape and K split that finish soonest under a cost model in
+    // microseconds.  Per variant and number r of workgroups resident on a CU, measured on MI355X
+    // (K = 1024 and 8192 on shapes of exactly r workgroups per CU): the time in which all r advance
+    // one K block, and the fixed time of a round (prologue, output, drain).  Workgroups are dealt in
+    // rounds of (CUs x the most that fit a CU); a last partial round runs with fewer per CU.  A K
+    // split adds the fp32 partial planes (written and read back, mostly through the 256 MB cache) and the
+    // reduce launch.
+    struct Cand { int variant; int rmax; double t_block[3], t_fixed[3]; };
+    const Cand cands[5] = {
+        {FP8BS_VARIANT_T256x256, 1, {1.87, 0, 0}, {6.8, 0, 0}},
+        {FP8BS_VARIANT_T256x192, 1, {1.45, 0, 0}, {6.0, 0, 0}},
+        {FP8BS_VARIANT_T256x128S3, 1, {1.18, 0, 0}, {4.2, 0, 0}},
+        {FP8BS_VARIANT_T128x128, 2, {0.89, 1.34, 0}, {3.1, 4.8, 0}},
+        {FP8BS_VARIANT_T64x128, 3, {0.70, 1.04, 1.39}, {1.9, 2.3, 3.6}},
+    };
+    const int splits[6] = {1, 2, 3, 4, 6, 8};
+    int best_variant = 0, best_split = 1; double best_cost = 0;
+    for (const Cand& c : cands) {
+        VariantInfo vi{};
+        variant_info(c.variant, &vi);
+        const long tiles = cdiv(m, vi.bm) * cdiv(n, vi.bn);
+        for (int s : splits) {
+            if (s > 1 && kbt / s < 4) continue;                  // keep at least 4 K blocks per workgroup
+            const long wgs = tiles * s, per_round = (long)num_cus * c.rmax;
+            const long full = wgs / per_round, rem = wgs % per_round;
+            const double kb = (double)cdiv(kbt, s);
+            double cost = (double)full * (c.t_fixed[c.rmax - 1] + kb * c.t_block[c.rmax - 1]);
+            if (rem) {
+                const long r = cdiv(rem, num_cus);
+                cost += c.t_fixed[r - 1] + kb * c.t_block[r - 1];
             }
+            if (s > 1) cost += 2.0 + 8.0 * s * (double)m * (double)n / 8.0e6;
+            if (best_variant == 0 || cost < best_cost) { best_variant = c.variant; best_split = s; best_cost = cost; }
         }
-        fill_plan(m, n, k, best_variant, best_split, out);
-        return;
     }
-    {
-        // Bandwidth-bound family: stream B once with the 64x144 ring kernel.  Pick the K split that
-        // minimises (rounds over the CUs) x (K blocks per workgroup) x (bytes of B per workgroup and
-        // K block) plus the fp32 partial planes the split writes and reads back.
-        long tiles = cdiv(m, 64) * cdiv(n, 144);
-        double best = 0; int best_s = 1;
-        for (int s = 1; s <= 8 && s <= kbt; s++) {
-            double t_main = (double)cdiv(tiles * s, num_cus) * (double)cdiv(kbt, s) * 144.0 * 128.0;
-            double t_red = s > 1 ? 8.0 * s * (double)m * (double)n / num_cus : 0.0;
-            if (s == 1 || t_main + t_red < best) { best = t_main + t_red; best_s = s; }
-        }
-        fill_plan(m, n, k, FP8BS_VARIANT_SKINNY64x144, best_s, out);
+    fill_plan(m, n, k, best_variant, best_split, out);
+}
+
+// The streaming kernel with the K split that fills the CUs (m a multiple of four).
+void choose_streaming(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
+    if (num_cus <= 0) num_cus = 256;
+    int kbt = k / KBLK;
+    // Bandwidth-bound family: stream B once with the 64x144 ring kernel.  Pick the K split that
+    // minimises (rounds over the CUs) x (K blocks per workgroup) x (bytes of B per workgroup and
+    // K block) plus the fp32 partial planes the split writes and reads back.
+    long tiles = cdiv(m, 64) * cdiv(n, 144);
+    double best = 0; int best_s = 1;
+    for (int s = 1; s <= 8 && s <= kbt; s++) {
+        double t_main = (double)cdiv(tiles * s, num_cus) * (double)cdiv(kbt, s) * 144.0 * 128.0;
+        double t_red = s > 1 ? 8.0 * s * (double)m * (double)n / num_cus : 0.0;
+        if (s == 1 || t_main + t_red < best) { best = t_main + t_red; best_s = s; }
+    }
+    fill_plan(m, n, k, FP8BS_VARIANT_SKINNY64x144, best_s, out);
+}
+
+// Shape-family rule.  n not a multiple of 8 -> generic kernel.  A few rows against a very large B -> the
+// streaming kernel (on padded copies of a / a_scale if m % 4 != 0).  Everything else -> the tiled kernel.
+void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
+    if (!vector_shape(n)) {
+        fill_plan(m, n, k, FP8BS_VARIANT_GENERIC, 1, out);
+    } else if (streaming_shape(m, n, k)) {
+        const int mp = (m + 3) & ~3;
+        choose_streaming(mp, n, k, num_cus, out);
+        if (mp != m) out->workspace_bytes += pad_bytes(k, mp);
+    } else {
+        choose_tiled(m, n, k, num_cus, out);
     }
 }
+
+bool is_streaming_variant(int v) { return v == FP8BS_VARIANT_SKINNY64x144 || v == FP8BS_VARIANT_SKINNY64x256 || v == FP8BS_VARIANT_SKINNY64x288; }
 
 int check_common(const void* a, const void* b, const float* as, const float* bs, void* c, int m, int n, int k) {
     if (m < 0 || n < 0 || k < 0 || (k % KBLK) != 0) return FP8BS_ERR_BAD_SHAPE;
@@ -225,46 +215,36 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
         if (variant != FP8BS_VARIANT_AUTO && variant != FP8BS_VARIANT_GENERIC) return FP8BS_ERR_BAD_VARIANT;
         variant = FP8BS_VARIANT_GENERIC;
     }
-    int m_main = m;                                    // rows the planned kernel computes
-    if (variant == FP8BS_VARIANT_AUTO && split_k == 0 && (m % 4) != 0 && m <= PAD_MAX_ROWS && (n % 8) == 0 && k > 0) {
-        // padded copies of a / a_scale at the head of the workspace, then the kernel planned for the padded
-        // row count; without enough workspace the two-launch scheme below (m >= 4) or the generic kernel
-        const int mp = (m + 3) & ~3;
-        choose(mp, n, k, 0, &plan);
-        const uint64_t pad = pad_bytes(k, mp);
-        const uint64_t planes = plan.split_k > 1 ? (uint64_t)plan.split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
-        if (ws && ws_bytes >= pad + planes) {
-            uint8_t* ap = (uint8_t*)ws;
-            float* asp = (float*)(ap + (size_t)k * mp);
-            if (fp8bs::launch_pad_rows((const uint8_t*)a, a_scale, ap, asp, m, mp, k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
-            fp8bs::GemmArgs g{};
-            g.a = ap; g.b = (const uint8_t*)b; g.as = asp; g.bs = b_scale;
-            g.c = (uint16_t*)c; g.ws = (float*)((uint8_t*)ws + pad); g.row_offsets = nullptr;
-            g.m = m; g.n = n; g.k = k; g.lda = mp; g.nb = (n + 127) / 128;
-            g.split_k = plan.split_k; g.kb_per_split = (int)cdiv(k / KBLK, plan.split_k); g.band_h = 4;
-            const int mode = plan.split_k > 1 ? 1 : 0;
-            if (fp8bs::launch_gemm(plan.variant, mode, g, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
-            if (mode == 1 && fp8bs::launch_splitk_reduce(g.ws, g.c, (size_t)m * n, plan.split_k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
-            return FP8BS_OK;
-        }
-        if (m < 4) variant = FP8BS_VARIANT_GENERIC;
-    }
+    bool padded = false;        // the streaming kernel runs on padded copies of a / a_scale in the workspace
     if (variant == FP8BS_VARIANT_AUTO) {
         choose(m, n, k, 0, &plan);
-        if (plan.variant != FP8BS_VARIANT_GENERIC && (m % 4) != 0) m_main = m & ~3;
-        if (split_k > 0) fill_plan(m_main, n, k, plan.variant, split_k, &plan);
+        if (is_streaming_variant(plan.variant) && (m % 4) != 0) {
+            const uint64_t planes = plan.split_k > 1 ? (uint64_t)plan.split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
+            if (split_k == 0 && ws && ws_bytes >= pad_bytes(k, (m + 3) & ~3) + planes) padded = true;
+            else choose_tiled(m, n, k, 0, &plan);     // no room for the copies (or a forced split): the tiled kernels take any m
+        }
+        if (split_k > 0) fill_plan(m, n, k, plan.variant, split_k, &plan);
     } else {
         VariantInfo vi{};
         if (!variant_info(variant, &vi)) return FP8BS_ERR_BAD_VARIANT;
-        if (variant != FP8BS_VARIANT_GENERIC && !vector_shape(m, n)) return FP8BS_ERR_BAD_VARIANT;
+        if (variant != FP8BS_VARIANT_GENERIC && !vector_shape(n)) return FP8BS_ERR_BAD_VARIANT;
+        if (is_streaming_variant(variant) && (m % 4) != 0) return FP8BS_ERR_BAD_VARIANT;
         fill_plan(m, n, k, variant, split_k > 0 ? split_k : 1, &plan);
     }
-    if (plan.split_k > 1 && (!ws || ws_bytes < (uint64_t)plan.split_k * (uint64_t)m_main * (uint64_t)n * 4u)) return FP8BS_ERR_WORKSPACE;
+    const int mp = (m + 3) & ~3;
+    const uint64_t pad = padded ? pad_bytes(k, mp) : 0u;
+    if (plan.split_k > 1 && (!ws || ws_bytes < pad + (uint64_t)plan.split_k * (uint64_t)m * (uint64_t)n * 4u)) return FP8BS_ERR_WORKSPACE;
 
     fp8bs::GemmArgs g{};
     g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.as = a_scale; g.bs = b_scale;
     g.c = (uint16_t*)c; g.ws = (float*)ws; g.row_offsets = nullptr;
-    g.m = m_main; g.n = n; g.k = k; g.lda = m; g.nb = (n + 127) / 128;
+    g.m = m; g.n = n; g.k = k; g.lda = m; g.nb = (n + 127) / 128;
+    if (padded) {
+        uint8_t* ap = (uint8_t*)ws;
+        float* asp = (float*)(ap + (size_t)k * mp);
+        if (fp8bs::launch_pad_rows((const uint8_t*)a, a_scale, ap, asp, m, mp, k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
+        g.a = ap; g.as = asp; g.lda = mp; g.ws = (float*)((uint8_t*)ws + pad);
+    }
     g.split_k = plan.split_k;
     g.kb_per_split = (int)cdiv(k / KBLK, plan.split_k);
     g.band_h = 4;
@@ -272,20 +252,7 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
     int mode = plan.split_k > 1 ? 1 : 0;
     if (fp8bs::launch_gemm(plan.variant, mode, g, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
     if (mode == 1) {
-        if (fp8bs::launch_splitk_reduce(g.ws, g.c, (size_t)m_main * n, plan.split_k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
-    }
-    if (m_main < m) {
-        // the last four rows (one to three of them new): same operands, shifted to row m - 4; the
-        // workspace is free again once the launches above have been queued on the same stream
-        fp8bs_plan_t tp{};
-        choose(4, n, k, 0, &tp);
-        if (tp.split_k > 1 && (!ws || ws_bytes < tp.workspace_bytes)) fill_plan(4, n, k, tp.variant, 1, &tp);
-        fp8bs::GemmArgs t = g;
-        t.a += m - 4; t.as += m - 4; t.c += (size_t)(m - 4) * n; t.row0 = m - 4;
-        t.m = 4; t.split_k = tp.split_k; t.kb_per_split = (int)cdiv(k / KBLK, tp.split_k);
-        const int tmode = tp.split_k > 1 ? 1 : 0;
-        if (fp8bs::launch_gemm(tp.variant, tmode, t, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
-        if (tmode == 1 && fp8bs::launch_splitk_reduce(t.ws, t.c, (size_t)4 * n, tp.split_k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
+        if (fp8bs::launch_splitk_reduce(g.ws, g.c, (size_t)m * n, plan.split_k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
     }
     return FP8BS_OK;
 }
@@ -309,7 +276,7 @@ int fp8bs_gemm_grouped_ex(const void* a, const void* b, const float* a_scale, co
     g.c = (uint16_t*)c; g.ws = nullptr; g.row_offsets = row_offsets;
     g.m = total_rows; g.n = n; g.k = k; g.lda = total_rows; g.nb = (n + 127) / 128;
     g.split_k = 1; g.kb_per_split = k / KBLK; g.band_h = 4; g.num_experts = num_experts;
-    const bool vector_ok = k != 0 && vector_shape(total_rows, n) && vector_aligned(a, b, c, nullptr);
+    const bool vector_ok = k != 0 && vector_shape(n) && vector_aligned(a, b, c, nullptr);
     if (variant == FP8BS_VARIANT_AUTO) {
         // The 256x256 tile for every routing: measured with 32 experts of 8 .. 1024 rows each (even and
         // random counts, n x k = 4096 x 7168 and 7168 x 2048) it is the fastest of the tiles throughout -
@@ -345,7 +312,7 @@ int fp8bs_gemm_silu_mul(const void* a, const void* b, const float* a_scale, cons
     g.split_k = 1; g.kb_per_split = k / KBLK; g.band_h = 4; g.num_experts = row_offsets ? num_experts : 0;
     g.epi = 1;
     // 16-byte stores of n/2-wide bf16 rows need n % 16 == 0
-    int variant = (k == 0 || !vector_shape(rows, n) || (n % 16) != 0 || !vector_aligned(a, b, h, nullptr)) ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
+    int variant = (k == 0 || !vector_shape(n) || (n % 16) != 0 || !vector_aligned(a, b, h, nullptr)) ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
     if (fp8bs::launch_gemm(variant, row_offsets ? 2 : 0, g, (hipStream_t)stream) != hipSuccess) return FP8BS_ERR_LAUNCH;
     return FP8BS_OK;
 }

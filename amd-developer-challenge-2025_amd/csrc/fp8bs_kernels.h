@@ -17,8 +17,7 @@ struct GemmArgs {
     float* ws;              // split-K partial planes [split_k][m][n]
     const int32_t* row_offsets;
     int m, n, k;
-    int lda;                // bytes per k row of a (the row count of the whole matrix)
-    int row0;               // a, as and c point at this row of the whole matrix (bounds of the loads end lda*k - row0 bytes after a)
+    int lda;                // bytes per k row of a (the row count of the whole matrix; the streaming kernels need a multiple of 4)
     int nb;                 // ceil(n / 128)
     int split_k, kb_per_split;
     int band_h;             // tile rows per band of the tile walk

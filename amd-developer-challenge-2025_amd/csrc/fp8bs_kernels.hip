@@ -168,6 +168,30 @@ __device__ __forceinline__ int stored_to_chunk(int st, int swz) {
     else { int x = st - swz; return x < 0 ? x + CPR : x; }
 }
 
+// Repair of the last bytes of a (see the main kernel).  cand*: bit 31 = the byte is lost, bits 29-30 = its
+// k row inside the last K block minus 125, bits 0-28 = its row; bits 8-31 of a_last = the bytes themselves.
+// stage_a: the A tile of the tile's last K block, m0 its first row, spare: a byte of LDS nobody reads.
+// Called by every wave right behind the barrier that publishes that block; ends with a second barrier.
+// No control flow: a store that does not apply goes to the spare byte.  (A branch at this place, in the
+// middle of a K block's step sequence, makes the compiler move the folds of the MFMAs before it below
+// it, which costs some thirty registers.)
+template <int BM, int CPR_A>
+__device__ __forceinline__ void patch_a_tail(unsigned char* stage_a, unsigned char* spare, bool enable, int m0,
+                                             uint32_t cand0, uint32_t cand1, uint32_t cand2, uint32_t a_last, int tid) {
+    const uint32_t cand[3] = {cand0, cand1, cand2};
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+        const int rt = (int)(cand[c] & 0x1FFFFFFFu) - m0;                 // row inside the tile
+        const int kl = KBLK - 3 + (int)((cand[c] >> 29) & 3u);            // k row inside the last block
+        const int rc = rt & (BM - 1);                                     // in range whatever rt is
+        unsigned char* dst = stage_a + kl * BM + (chunk_to_stored<CPR_A>(rc >> 4, swz_of_krow<CPR_A>(kl)) << 4) + (rc & 15);
+        int apply = (enable && (cand[c] >> 31) != 0 && rt >= 0 && rt < BM && tid == 0) ? 1 : 0;
+        asm volatile("" : "+v"(apply));       // opaque to the optimiser: a select follows, never a branch
+        *(apply != 0 ? dst : spare) = (unsigned char)(a_last >> (8 * (c + 1)));
+    }
+    __syncthreads();
+}
+
 // EPI 0: plain bf16 output.  EPI 1: gate/up pairs - column 2i is gate_i, column 2i+1 is up_i - are
 // combined to silu(gate_i) * up_i in fp32 and the output has n/2 columns (role of the fp16 layer's
 // re_silu_mul_kernel, 2-amd-moe/amd-moe-submission.py:366-407, fused into the GEMM as in
@@ -177,7 +201,9 @@ __device__ __forceinline__ float silu_mul(float gate, float up) {
     return gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * gate)) * up;
 }
 
-template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0, int NSTAGE = 2>
+// ATAIL: lda is not a multiple of four; the kernel then repairs the last bytes of a in LDS (one more
+// barrier per tile), see below.
+template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0, int NSTAGE = 2, bool ATAIL = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64)
 void gemm_tr_kernel(const GemmArgs p) {
     using C = TileCfg<BM, BN, WM, WN, MODE, NSTAGE>;
@@ -278,7 +304,7 @@ void gemm_tr_kernel(const GemmArgs p) {
     };
 
     // ---- buffer resources: out-of-range lanes read zeros instead of faulting -------------------
-    const uint32_t a_bytes = (uint32_t)p.k * (uint32_t)p.lda - (uint32_t)p.row0;
+    const uint32_t a_bytes = (uint32_t)p.k * (uint32_t)p.lda;
     const uint32_t b_bytes = (uint32_t)p.k * (uint32_t)p.n;
     __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, a_bytes, 0x00020000);
 
@@ -343,7 +369,7 @@ void gemm_tr_kernel(const GemmArgs p) {
         c.b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.bptr, 0, b_bytes, 0x00020000);
         c.sc_rsrc = __builtin_amdgcn_make_buffer_rsrc(sc_is_b ? (void*)t.bsptr : (void*)p.as, 0,
                                                       sc_is_b ? (uint32_t)(p.k / KBLK) * (uint32_t)p.nb * 4u
-                                                              : ((uint32_t)(p.k / KBLK) * (uint32_t)p.lda - (uint32_t)p.row0) * 4u, 0x00020000);
+                                                              : (uint32_t)(p.k / KBLK) * (uint32_t)p.lda * 4u, 0x00020000);
         return c;
     };
     const uint32_t a_kstep = (uint32_t)KBLK * (uint32_t)p.lda, b_kstep = (uint32_t)KBLK * (uint32_t)p.n;
@@ -406,6 +432,31 @@ void gemm_tr_kernel(const GemmArgs p) {
     const int as_lane_off = C::A_BYTES + C::B_BYTES + (wave_m * WM + i16) * 4;
     const int bs_base = C::A_BYTES + C::B_BYTES + C::AS_AREA;     // slot i: b_scale of n block n0/128 + i
 
+    // ---- rows of a that are not a multiple of four --------------------------------------------------
+    // The buffer of a ends on a dword boundary (K is a multiple of 128), but with lda % 4 != 0 the copies
+    // fetch its last one to three bytes in dwords that start inside and end beyond it; the range check
+    // of a buffer load works on whole dwords and hands back zeros for those.  Every other byte of a
+    // arrives intact (a dword that crosses the end of a k row just runs on into the next one).  The
+    // workgroup whose tile holds those bytes writes them into LDS itself once the last K block has
+    // landed: they all lie in the last aligned dword of a.
+    const uint32_t a_end = (uint32_t)p.k * (uint32_t)p.lda;
+    const bool a_tail = ATAIL && (p.lda & 3) != 0 && p.k > 0;
+    // The three candidates (byte offsets a_end-3 .. a_end-1) are worked out once, here, where registers are
+    // plentiful, and kept in scalar registers: bit 31 = the byte is lost, bits 29-30 = its k row inside the
+    // last K block minus 125, bits 0-28 = its row; bits 8-31 of a_last = the three bytes themselves.
+    uint32_t cand0 = 0, cand1 = 0, cand2 = 0, a_last = 0;
+    if (a_tail) {
+        auto candidate = [&](uint32_t o) __attribute__((always_inline)) -> uint32_t {
+            const uint32_t krow = o / (uint32_t)p.lda, row = o - krow * (uint32_t)p.lda;
+            const bool lost = krow * (uint32_t)p.lda + (row & ~3u) + 4u > a_end;          // its dword crosses the end
+            return lost ? (0x80000000u | ((krow - ((uint32_t)p.k - 3u)) << 29) | row) : 0u;
+        };
+        cand0 = candidate(a_end - 3); cand1 = candidate(a_end - 2); cand2 = candidate(a_end - 1);
+        a_last = *(const uint32_t*)(p.a + (a_end - 4));
+    }
+    // (the load is consumed here, not inside the K loop)
+    cand0 = __builtin_amdgcn_readfirstlane(cand0); cand1 = __builtin_amdgcn_readfirstlane(cand1);
+    cand2 = __builtin_amdgcn_readfirstlane(cand2); a_last = __builtin_amdgcn_readfirstlane(a_last);
     Tile cur = pick_tile(0);
     if (!cur.valid) return;
     CopyPlan cp = copy_plan(cur);
@@ -431,6 +482,7 @@ void gemm_tr_kernel(const GemmArgs p) {
         for (int u = 0; u < C::NT; u++) acc[t][u] = (v4f){0.f, 0.f, 0.f, 0.f};
 
     const int nkb = kb_end - kb_begin;
+    const bool patch_tile = a_tail && kb_end * KBLK == p.k;       // this tile's last K block is the last of a
     if (nkb > 0) {
         constexpr int STEPS = C::MT * C::NT;
         constexpr int LAG = 3, RING = 4;      // fold the result of step s-LAG while step s runs
@@ -463,6 +515,7 @@ void gemm_tr_kernel(const GemmArgs p) {
             else { if (sb) wait_vmcnt<EPI_STORES>(); else wait_vmcnt<0>(); }
         }
         __syncthreads();
+        if (ATAIL && nkb == 1) patch_a_tail<BM, C::CPR_A>(lds, lds + C::STAGE_BYTES - 1, patch_tile, m0, cand0, cand1, cand2, a_last, tid);
         if (nkb > NSTAGE - 1) {
             [&]<int... Q>(std::integer_sequence<int, Q...>) {
                 (issue_one(cp, NSTAGE - 1, NSTAGE - 1, std::integral_constant<int, Q>{}), ...);
@@ -490,6 +543,7 @@ void gemm_tr_kernel(const GemmArgs p) {
             constexpr bool HAS_NEXT = decltype(h1_tag)::value;                                              // block j+1 exists
             constexpr bool HAS_EARLY = NSTAGE == 2 ? decltype(h1_tag)::value : decltype(h2_tag)::value;    // block j+NSTAGE-1 exists
             constexpr bool HAS_LATE = NSTAGE == 2 ? decltype(h2_tag)::value : decltype(h3_tag)::value;     // block j+NSTAGE exists
+            constexpr bool LANDS_LAST = decltype(h1_tag)::value && !decltype(h2_tag)::value;               // block j+1 is the tile's last
             const int cur_stage = NSTAGE == 2 ? (j & 1) : j % NSTAGE;
             const int next_stage = cur_stage + 1 == NSTAGE ? 0 : cur_stage + 1;
             const int early_stage = NSTAGE == 2 ? next_stage : (next_stage + 1 == NSTAGE ? 0 : next_stage + 1);
@@ -509,6 +563,7 @@ void gemm_tr_kernel(const GemmArgs p) {
                 }
                 wait_next_block();
                 __syncthreads();
+                if constexpr (ATAIL && LANDS_LAST) patch_a_tail<BM, C::CPR_A>(lds + next_stage * C::STAGE_BYTES, lds + cur_stage * C::STAGE_BYTES + C::STAGE_BYTES - 1, patch_tile, m0, cand0, cand1, cand2, a_last, tid);
                 if constexpr (HAS_LATE) {
                     [&]<int... Q>(std::integer_sequence<int, Q...>) {
                         (issue_one(cp, cur_stage, j + NSTAGE, std::integral_constant<int, Q>{}), ...);
@@ -541,6 +596,7 @@ void gemm_tr_kernel(const GemmArgs p) {
                         // block is complete in the other stage and this stage may be overwritten.
                         wait_next_block();
                         __syncthreads();
+                        if constexpr (ATAIL && LANDS_LAST) patch_a_tail<BM, C::CPR_A>(lds + next_stage * C::STAGE_BYTES, lds + cur_stage * C::STAGE_BYTES + C::STAGE_BYTES - 1, patch_tile, m0, cand0, cand1, cand2, a_last, tid);
                     }
                     const v4f z = {0.f, 0.f, 0.f, 0.f};
                     ring[s % RING] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(breg[u & 1], areg[t], z, 0, 0, 0, 0, 0, 0);
@@ -766,8 +822,8 @@ void gemm_skinny_kernel(const GemmArgs p) {
     const int nkb = kb_end - kb_begin;
     const int nb0 = n0 / 128;
 
-    const uint32_t a_bytes = (uint32_t)p.k * (uint32_t)p.lda - (uint32_t)p.row0, b_bytes = (uint32_t)p.k * (uint32_t)p.n;
-    const uint32_t as_bytes = ((uint32_t)kbt * (uint32_t)p.lda - (uint32_t)p.row0) * 4u, bs_bytes = (uint32_t)kbt * (uint32_t)p.nb * 4u;
+    const uint32_t a_bytes = (uint32_t)p.k * (uint32_t)p.lda, b_bytes = (uint32_t)p.k * (uint32_t)p.n;
+    const uint32_t as_bytes = (uint32_t)kbt * (uint32_t)p.lda * 4u, bs_bytes = (uint32_t)kbt * (uint32_t)p.nb * 4u;
 
     // ---- copy plan.  The one-KiB copies of a block are numbered I = 4q + wave, q = 0..COPIES-1:
     //      I < A_COPIES the A tile, then B_COPIES of the B tile (copy Ib fills B chunks 64*Ib ..), then the
@@ -1004,9 +1060,11 @@ void gemm_generic_kernel(const GemmArgs p) {
 template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0, int NSTAGE = 2>
 static hipError_t launch_tr(const GemmArgs& a, dim3 grid, hipStream_t stream) {
     using C = TileCfg<BM, BN, WM, WN, MODE, NSTAGE>;
-    auto kern = gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI, NSTAGE>;
-    static int raised[MAX_DEVICES];
-    hipError_t e = raise_lds_limit((const void*)kern, C::LDS_BYTES, raised);
+    // rows of a that are not a multiple of four: the instantiation that repairs the last bytes of a
+    const bool atail = (a.lda & 3) != 0;
+    void (*kern)(const GemmArgs) = atail ? gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI, NSTAGE, true> : gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI, NSTAGE, false>;
+    static int raised[2][MAX_DEVICES];
+    hipError_t e = raise_lds_limit((const void*)kern, C::LDS_BYTES, raised[atail ? 1 : 0]);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, grid, dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
     return hipGetLastError();

@@ -34,12 +34,12 @@ def test_plan_shape_families(pkg):
     assert p.workspace_bytes == p.split_k * 64 * 18432 * 4 == pkg.workspace_bytes(64, 18432, 7168)
     p = pkg.plan(130, 190, 256)                         # n not a multiple of 8 -> generic kernel
     assert p.variant == 1 and p.split_k == 1
-    p, q = pkg.plan(130, 192, 256), pkg.plan(132, 192, 256)   # m % 4 != 0, few rows: the plan of 132 rows on padded copies of a / a_scale
-    assert p.variant == q.variant != 1 and p.split_k == q.split_k and p.workspace_bytes == q.workspace_bytes + 35072   # 256*132 + 2*132*4 -> 35072
-    p, q = pkg.plan(4095, 512, 256), pkg.plan(4092, 512, 256) # many rows: the plan of the first 4092 rows, the last four in a second launch
-    assert p.variant == q.variant != 1 and p.split_k == q.split_k and p.workspace_bytes >= q.workspace_bytes
-    p, q = pkg.plan(3, 192, 256), pkg.plan(4, 192, 256)       # 1..3 rows: four-row copies in the workspace
-    assert p.variant == q.variant != 1 and p.workspace_bytes == q.workspace_bytes + 1280   # 4*256 + 16*2 -> 1280
+    for m in (130, 4095, 3, 1):                               # any m: the tiled kernels, one launch, nothing extra in the workspace
+        p, q = pkg.plan(m, 192, 256), pkg.plan((m + 3) & ~3, 192, 256)
+        assert p.variant == q.variant and p.variant not in (1, 6, 7, 8) and p.split_k == q.split_k
+        assert p.workspace_bytes == (p.split_k * m * 192 * 4 if p.split_k > 1 else 0)
+    p, q = pkg.plan(3, 18432, 7168), pkg.plan(4, 18432, 7168) # a few rows against a large b: the streaming kernel on four-row copies in the workspace
+    assert p.variant == q.variant == 6 and p.workspace_bytes == q.workspace_bytes + ((4 * 7168 + 16 * 56 + 255) & ~255)   # 4 K + 16 K/128 bytes, rounded up to 256
     assert pkg.plan(3, 190, 256).variant == 1
     p = pkg.plan(256, 512, 1024)                        # small: one of the sub-256 tiles, never the scalar kernel
     assert p.variant in (3, 4, 10) and p.split_k >= 1 and p.split_k <= 8
@@ -62,10 +62,12 @@ def test_plan_streaming_kernel_only_for_few_rows_against_a_large_b(pkg):
         p = pkg.plan(m, n, k)
         assert (p.variant in (6, 7, 8)) == streaming, (m, n, k, p.variant)
         assert p.variant != 1
-        if m % 4 == 0:
+        if m % 4 == 0 or not streaming:
             assert p.workspace_bytes == (p.split_k * m * n * 4 if p.split_k > 1 else 0)
-    # one to three rows take the plan of four rows plus the padded copies
-    assert pkg.plan(1, 18432, 7168).variant == pkg.plan(4, 18432, 7168).variant == 6
+    # rows that are not a multiple of four: the streaming plan of the padded row count plus the padded copies
+    for m in (1, 5, 63):
+        p, q = pkg.plan(m, 18432, 7168), pkg.plan((m + 3) & ~3, 18432, 7168)
+        assert p.variant == q.variant == 6 and p.split_k == q.split_k and p.workspace_bytes > q.workspace_bytes
 
 
 def test_plan_rejects_bad_shapes(pkg):
@@ -86,7 +88,8 @@ def test_argument_errors_are_reported_before_any_launch(pkg):
     assert lib.fp8bs_gemm(one, one, one, one, one, None, 0, 0, 16, 128, None) == 0       # empty: nothing to do
     assert lib.fp8bs_gemm(one, one, one, one, one, None, 0, 1 << 20, 16, 1 << 13, None) == 4   # 2^33 bytes of a
     assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 16, 16, 128, 99, 1, None) == 7
-    assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 130, 16, 128, 2, 1, None) == 7  # tiled variant needs m%16==0
+    assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 128, 20, 128, 2, 1, None) == 7  # the vector kernels need n % 8 == 0
+    assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 130, 16, 128, 6, 1, None) == 7  # the streaming kernels need m % 4 == 0
     assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 64, 256, 1024, 4, 4, None) == 3 # split-K without workspace
     assert lib.fp8bs_gemm_grouped(one, one, one, one, one, None, 4, 16, 16, 128, None) == 1
     assert lib.fp8bs_gemm_grouped(one, one, one, one, one, one, 0, 16, 16, 128, None) == 6

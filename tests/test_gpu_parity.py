@@ -81,7 +81,7 @@ def test_every_variant_and_split_on_config1(pkg, oracle, dev, variant, split_k):
                                    (132, 200, 256), (20, 24, 128), (516, 264, 384), (268, 2104, 256),
                                    (4095, 512, 256), (1021, 264, 384), (131, 1024, 512), (61, 2048, 1024), (5, 16, 128),
                                    (1, 2048, 1024), (2, 264, 384), (3, 18432, 512), (5, 18432, 512), (1030, 264, 256), (2050, 136, 384),
-                                   (1023, 8, 128), (67, 2112, 640)])
+                                   (1023, 8, 128), (67, 2112, 640), (7, 64, 128), (2, 8, 256), (255, 256, 128), (257, 192, 384), (513, 136, 1024)])
 def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
     """N tails (2112 = 16*128 + 64), tiles larger than the matrix, rows and columns that end inside a
     16-byte chunk (m % 4 == 0, n % 8 == 0: still the vector kernels), shapes only the generic kernel takes."""
@@ -91,16 +91,21 @@ def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
     _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d" % (m, n, k))
     if n % 8 == 0:
         assert pkg.plan(m, n, k).variant != 1                   # any m: the vector kernels, in two launches if m % 4 != 0
-    if m % 4 == 0 and n % 8 == 0:
-        for variant in (2, 3, 4, 5, 6, 7, 8, 9, 10):
+    if n % 8 == 0:
+        # every tile takes any m (the last bytes of a are repaired in LDS); the streaming kernels m % 4 == 0
+        for variant in (2, 3, 4, 5, 9, 10) + ((6, 7, 8) if m % 4 == 0 else ()):
             out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1)
             _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d" % (m, n, k, variant))
+        if k >= 512:
+            out = pkg.custom_kernel(_to(cpu, dev), variant=4, split_k=2)        # the repair happens in the last split only
+            _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant 4 split 2" % (m, n, k))
 
 
 @pytest.mark.parametrize("m,n,k,variant", [(8192, 8192, 256, 2), (8188, 4104, 128, 0), (4096, 8192, 384, 5),
                                            (8192, 4096, 256, 3), (4096, 4096, 256, 4),
                                            (8192, 8256, 256, 9), (4100, 2112, 384, 9), (4096, 6336, 128, 9),
-                                           (8192, 8192, 128, 10), (8192, 4096, 256, 10), (4100, 8200, 384, 10), (4096, 4096, 512, 10)])
+                                           (8192, 8192, 128, 10), (8192, 4096, 256, 10), (4100, 8200, 384, 10), (4096, 4096, 512, 10),
+                                           (8191, 2048, 128, 2), (4095, 2112, 384, 0), (4097, 4096, 256, 3), (4091, 4104, 128, 4), (2049, 8192, 256, 10)])
 def test_many_tiles_per_workgroup_against_the_scalar_kernel(pkg, oracle, dev, m, n, k, variant):
     """Short K and a large output: every persistent workgroup walks many tiles, so the hand-over between
     tiles (next tile's first block issued ahead of the output stores, counted wait) carries the result.
@@ -149,8 +154,8 @@ def test_repeated_calls_skip_the_checks_but_not_after_a_change(pkg, oracle, dev)
 
 
 def test_seeded_random_shapes_through_the_planner(pkg, oracle, dev):
-    """40 seeded shapes on the 4 x 8 grid of the vector kernels, whatever the planner picks for each
-    (tile shape, K split, streaming kernel), plus one forced K split per shape."""
+    """40 seeded shapes with n on the 8-column grid of the vector kernels and any m, whatever the planner
+    picks for each (tile shape, K split, streaming kernel), plus one forced K split per shape."""
     rng = np.random.default_rng(20259)
     cfg = pkg.inputs.CONFIGS[2]                                   # outlier activations, small weights
     seen = set()
@@ -161,6 +166,9 @@ def test_seeded_random_shapes_through_the_planner(pkg, oracle, dev):
             m = int(rng.choice([4, 8, 12, 16])) * int(rng.integers(1, 60)) if i % 3 else 4 * int(rng.integers(1, 40))
             n = 8 * int(rng.integers(1, 140))
         k = 128 * int(rng.integers(1, 13))
+        if i % 2:
+            m -= int(rng.integers(1, 4))                          # half of the shapes off the 4-row grid
+            m = max(m, 1)
         cpu = pkg.inputs.make_dense(cfg, m=m, n=n, k=k)
         ref = oracle.ref_kernel(cpu)
         plan = pkg.plan(m, n, k)
@@ -168,9 +176,11 @@ def test_seeded_random_shapes_through_the_planner(pkg, oracle, dev):
         out = pkg.custom_kernel(_to(cpu, dev))
         _check(oracle, out, ref, "shape %dx%dx%d planned variant %d split %d" % (m, n, k, plan.variant, plan.split_k))
         split = int(rng.integers(2, 6))
+        if plan.variant in (6, 7, 8) and m % 4:
+            continue                                              # the streaming kernels cannot be forced on such an m
         out = pkg.custom_kernel(_to(cpu, dev), variant=plan.variant, split_k=split)
         _check(oracle, out, ref, "shape %dx%dx%d variant %d forced split %d" % (m, n, k, plan.variant, split))
-    assert len({v for v, _ in seen}) >= 4, "the draw should reach several kernel variants: %s" % sorted(seen)
+    assert len({v for v, _ in seen}) >= 3 and any(s for _, s in seen), "the draw should reach several tiles and a K split: %s" % sorted(seen)
 
 
 def _shifted(t, nbytes):
@@ -198,6 +208,24 @@ def test_pointers_off_the_16_byte_grid_take_the_generic_kernel(pkg, oracle, dev,
     _check(oracle, out, oracle.ref_kernel(cpu), "misaligned " + which)
     with pytest.raises(RuntimeError):
         pkg.custom_kernel((a, b, a_scale, b_scale, c), variant=2, split_k=1)     # a forced vector kernel is refused
+
+
+@pytest.mark.parametrize("m,n,k", [(5, 264, 384), (3, 264, 384), (131, 1024, 256), (1027, 136, 256)])
+def test_rows_not_a_multiple_of_four_without_a_workspace(pkg, oracle, dev, m, n, k):
+    """Through the C ABI with no workspace at all (the plans have no K split at these sizes).  Same results
+    as with a workspace."""
+    cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[2], m=m, n=n, k=k)
+    a, b, a_scale, b_scale, c = _to(cpu, dev)
+    assert pkg.plan(m, n, k).split_k == 1
+    lib = pkg._lib.load()
+    c.fill_(float("nan"))
+    st = lib.fp8bs_gemm(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(), c.data_ptr(), None, 0, m, n, k,
+                        torch.cuda.current_stream().cuda_stream)
+    assert st == 0, pkg._lib.load().fp8bs_strerror(st)
+    torch.cuda.synchronize()
+    _check(oracle, c, oracle.ref_kernel(cpu), "no workspace %dx%dx%d" % (m, n, k))
+    with_ws = pkg.custom_kernel((a, b, a_scale, b_scale, torch.full_like(c, float("nan"))))
+    _check(oracle, with_ws, oracle.ref_kernel(cpu), "workspace %dx%dx%d" % (m, n, k))
 
 
 def test_empty_shapes(pkg, dev):
@@ -312,15 +340,12 @@ def test_grouped_every_element_against_the_scalar_kernel(pkg, dev):
 
 
 @pytest.mark.parametrize("variant", [2, 3, 4, 5, 9, 10])
-@pytest.mark.parametrize("tokens,experts,topk,n,k", [(96, 8, 2, 448, 384), (1024, 32, 8, 2112, 256), (40, 16, 1, 256, 128)])
+@pytest.mark.parametrize("tokens,experts,topk,n,k", [(96, 8, 2, 448, 384), (1024, 32, 8, 2112, 256), (40, 16, 1, 256, 128), (37, 8, 3, 264, 384), (341, 4, 1, 512, 128)])
 def test_grouped_with_every_tile_against_the_scalar_kernel(pkg, dev, variant, tokens, experts, topk, n, k):
     """Every tile shape in grouped mode: experts of a few rows, empty experts (40 tokens over 16 experts), expert boundaries inside a
     tile and inside a 16-row group, column tails.  Every element against the scalar kernel."""
     cfg = pkg.inputs.CONFIGS[4]
     data = list(_to(pkg.inputs.make_grouped(cfg, tokens=tokens, experts=experts, topk=topk, n=n, k=k), dev))
-    rows = data[0].shape[0]
-    if rows % 4:
-        pytest.skip("the vector kernels need a multiple of four rows")
     ref = pkg.grouped_kernel(tuple(data[:5]) + (torch.full_like(data[5], float("nan")),), variant=1).float()
     out = pkg.grouped_kernel(tuple(data[:5]) + (torch.full_like(data[5], float("nan")),), variant=variant).float()
     auto = pkg.grouped_kernel(tuple(data[:5]) + (torch.full_like(data[5], float("nan")),)).float()
