@@ -64,8 +64,10 @@ void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out)
 // of the workspace (k * mp bytes: the streaming kernels only ever see a few rows).
 uint64_t pad_bytes(int k, int mp) { return (((uint64_t)k * (uint64_t)mp + (uint64_t)(k / KBLK) * (uint64_t)mp * 4u) + 255u) & ~(uint64_t)255u; }
 
-// What the vector kernels need of a shape: rows of c (n bf16) that keep 16-byte stores aligned.  The
-// tiled kernels take any m (they repair the last bytes of a themselves), the streaming kernels m % 4 == 0.
+// Rows of c (n bf16) that keep 16-byte stores aligned: what the streaming kernels, the K split (its
+// reduction works on groups of eight outputs), the grouped walk and the fused epilogue need.  The tiled
+// kernels without a K split take any m and n (they repair the last bytes of a and b themselves and store
+// a row's last chunk of c in pieces); the streaming kernels also need m % 4 == 0.
 bool vector_shape(int n) { return (n % 8) == 0; }
 
 // The streaming kernel is kept for what it was built for: at most 64 rows against a B too large for the
@@ -75,8 +77,9 @@ bool vector_shape(int n) { return (n % 8) == 0; }
 // second row of tiles and reads B twice.
 bool streaming_shape(int m, int n, int k) { return m <= 64 && (double)n * (double)k >= 96.0e6; }
 
-// The tile shape and K split of the tiled MFMA kernel that finish soonest (any m).
+// The tile shape and K split of the tiled MFMA kernel that finish soonest (any m; any n without a split).
 void choose_tiled(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
+    const bool may_split = vector_shape(n);
     if (num_cus <= 0) num_cus = 256;
     int kbt = k / KBLK;
     // The tile shape and K split that finish soonest under a cost model in
@@ -101,7 +104,7 @@ void choose_tiled(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
         variant_info(c.variant, &vi);
         const long tiles = cdiv(m, vi.bm) * cdiv(n, vi.bn);
         for (int s : splits) {
-            if (s > 1 && kbt / s < 4) continue;                  // keep at least 4 K blocks per workgroup
+            if (s > 1 && (kbt / s < 4 || !may_split)) continue;  // keep at least 4 K blocks per workgroup
             const long wgs = tiles * s, per_round = (long)num_cus * c.rmax;
             const long full = wgs / per_round, rem = wgs % per_round;
             const double kb = (double)cdiv(kbt, s);
@@ -134,12 +137,10 @@ void choose_streaming(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     fill_plan(m, n, k, FP8BS_VARIANT_SKINNY64x144, best_s, out);
 }
 
-// Shape-family rule.  n not a multiple of 8 -> generic kernel.  A few rows against a very large B -> the
-// streaming kernel (on padded copies of a / a_scale if m % 4 != 0).  Everything else -> the tiled kernel.
+// Shape-family rule.  A few rows against a very large B -> the streaming kernel (on padded copies of
+// a / a_scale if m % 4 != 0).  Everything else -> the tiled kernel.
 void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
-    if (!vector_shape(n)) {
-        fill_plan(m, n, k, FP8BS_VARIANT_GENERIC, 1, out);
-    } else if (streaming_shape(m, n, k)) {
+    if (vector_shape(n) && streaming_shape(m, n, k)) {
         const int mp = (m + 3) & ~3;
         choose_streaming(mp, n, k, num_cus, out);
         if (mp != m) out->workspace_bytes += pad_bytes(k, mp);
@@ -223,11 +224,12 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
             if (split_k == 0 && ws && ws_bytes >= pad_bytes(k, (m + 3) & ~3) + planes) padded = true;
             else choose_tiled(m, n, k, 0, &plan);     // no room for the copies (or a forced split): the tiled kernels take any m
         }
+        if (split_k > 1 && !vector_shape(n)) return FP8BS_ERR_BAD_VARIANT;
         if (split_k > 0) fill_plan(m, n, k, plan.variant, split_k, &plan);
     } else {
         VariantInfo vi{};
         if (!variant_info(variant, &vi)) return FP8BS_ERR_BAD_VARIANT;
-        if (variant != FP8BS_VARIANT_GENERIC && !vector_shape(n)) return FP8BS_ERR_BAD_VARIANT;
+        if (variant != FP8BS_VARIANT_GENERIC && !vector_shape(n) && (is_streaming_variant(variant) || split_k > 1)) return FP8BS_ERR_BAD_VARIANT;
         if (is_streaming_variant(variant) && (m % 4) != 0) return FP8BS_ERR_BAD_VARIANT;
         fill_plan(m, n, k, variant, split_k > 0 ? split_k : 1, &plan);
     }

@@ -36,6 +36,7 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
@@ -168,28 +169,33 @@ __device__ __forceinline__ int stored_to_chunk(int st, int swz) {
     else { int x = st - swz; return x < 0 ? x + CPR : x; }
 }
 
-// Repair of the last bytes of a (see the main kernel).  cand*: bit 31 = the byte is lost, bits 29-30 = its
-// k row inside the last K block minus 125, bits 0-28 = its row; bits 8-31 of a_last = the bytes themselves.
-// stage_a: the A tile of the tile's last K block, m0 its first row, spare: a byte of LDS nobody reads.
-// Called by every wave right behind the barrier that publishes that block; ends with a second barrier.
-// No control flow: a store that does not apply goes to the spare byte.  (A branch at this place, in the
-// middle of a K block's step sequence, makes the compiler move the folds of the MFMAs before it below
-// it, which costs some thirty registers.)
-template <int BM, int CPR_A>
-__device__ __forceinline__ void patch_a_tail(unsigned char* stage_a, unsigned char* spare, bool enable, int m0,
-                                             uint32_t cand0, uint32_t cand1, uint32_t cand2, uint32_t a_last, int tid) {
+// Repair of the last bytes of a or b (see the main kernel).  cand[i]: bit 31 = the byte is lost, bits
+// 29-30 = its k row inside the last K block minus 125, bits 0-28 = its row (of a) or column (of b); bits
+// 8-31 of `last` = the bytes themselves.  tile: the operand's tile of the tile's last K block, x0 its first
+// row / column, spare: a byte of LDS nobody reads.  No control flow: a store that does not apply goes to
+// the spare byte.  (A branch at this place, in the middle of a K block's step sequence, makes the compiler
+// move the folds of the MFMAs before it below it, which costs some thirty registers.)
+template <int BX, int CPR>
+__device__ __forceinline__ void patch_tail_bytes(unsigned char* tile, unsigned char* spare, bool enable, int x0,
+                                                 uint32_t cand0, uint32_t cand1, uint32_t cand2, uint32_t last, int tid) {
     const uint32_t cand[3] = {cand0, cand1, cand2};
 #pragma unroll
     for (int c = 0; c < 3; c++) {
-        const int rt = (int)(cand[c] & 0x1FFFFFFFu) - m0;                 // row inside the tile
+        const int xt = (int)(cand[c] & 0x1FFFFFFFu) - x0;                 // row / column inside the tile
         const int kl = KBLK - 3 + (int)((cand[c] >> 29) & 3u);            // k row inside the last block
-        const int rc = rt & (BM - 1);                                     // in range whatever rt is
-        unsigned char* dst = stage_a + kl * BM + (chunk_to_stored<CPR_A>(rc >> 4, swz_of_krow<CPR_A>(kl)) << 4) + (rc & 15);
-        int apply = (enable && (cand[c] >> 31) != 0 && rt >= 0 && rt < BM && tid == 0) ? 1 : 0;
+        int xc = xt < 0 ? 0 : xt;                                         // in range whatever xt is
+        xc = xc < BX ? xc : BX - 1;
+        unsigned char* dst = tile + kl * BX + (chunk_to_stored<CPR>(xc >> 4, swz_of_krow<CPR>(kl)) << 4) + (xc & 15);
+        int apply = (enable && (cand[c] >> 31) != 0 && xt >= 0 && xt < BX && tid == 0) ? 1 : 0;
         asm volatile("" : "+v"(apply));       // opaque to the optimiser: a select follows, never a branch
-        *(apply != 0 ? dst : spare) = (unsigned char)(a_last >> (8 * (c + 1)));
+        *(apply != 0 ? dst : spare) = (unsigned char)(last >> (8 * (c + 1)));
     }
-    __syncthreads();
+}
+// The three candidates of an operand whose k rows are ld bytes long and whose buffer ends at `end`.
+__device__ __forceinline__ uint32_t tail_candidate(uint32_t o, uint32_t ld, uint32_t end, uint32_t k) {
+    const uint32_t krow = o / ld, x = o - krow * ld;
+    const bool lost = krow * ld + (x & ~3u) + 4u > end;                   // its dword crosses the end
+    return lost ? (0x80000000u | ((krow - (k - 3u)) << 29) | x) : 0u;
 }
 
 // EPI 0: plain bf16 output.  EPI 1: gate/up pairs - column 2i is gate_i, column 2i+1 is up_i - are
@@ -201,9 +207,10 @@ __device__ __forceinline__ float silu_mul(float gate, float up) {
     return gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * gate)) * up;
 }
 
-// ATAIL: lda is not a multiple of four; the kernel then repairs the last bytes of a in LDS (one more
-// barrier per tile), see below.
-template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0, int NSTAGE = 2, bool ATAIL = false>
+// TAILS: lda is not a multiple of four or n not a multiple of eight; the kernel then repairs the last
+// bytes of a and b in LDS (one more barrier per tile) and stores a row's last, partial 16-byte chunk of c
+// in pieces, see below.
+template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0, int NSTAGE = 2, bool TAILS = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64)
 void gemm_tr_kernel(const GemmArgs p) {
     using C = TileCfg<BM, BN, WM, WN, MODE, NSTAGE>;
@@ -432,31 +439,48 @@ void gemm_tr_kernel(const GemmArgs p) {
     const int as_lane_off = C::A_BYTES + C::B_BYTES + (wave_m * WM + i16) * 4;
     const int bs_base = C::A_BYTES + C::B_BYTES + C::AS_AREA;     // slot i: b_scale of n block n0/128 + i
 
-    // ---- rows of a that are not a multiple of four --------------------------------------------------
+    // ---- rows of a that are not a multiple of four, columns of b that are not ------------------------
     // The buffer of a ends on a dword boundary (K is a multiple of 128), but with lda % 4 != 0 the copies
     // fetch its last one to three bytes in dwords that start inside and end beyond it; the range check
     // of a buffer load works on whole dwords and hands back zeros for those.  Every other byte of a
     // arrives intact (a dword that crosses the end of a k row just runs on into the next one).  The
     // workgroup whose tile holds those bytes writes them into LDS itself once the last K block has
-    // landed: they all lie in the last aligned dword of a.
-    const uint32_t a_end = (uint32_t)p.k * (uint32_t)p.lda;
-    const bool a_tail = ATAIL && (p.lda & 3) != 0 && p.k > 0;
-    // The three candidates (byte offsets a_end-3 .. a_end-1) are worked out once, here, where registers are
-    // plentiful, and kept in scalar registers: bit 31 = the byte is lost, bits 29-30 = its k row inside the
-    // last K block minus 125, bits 0-28 = its row; bits 8-31 of a_last = the three bytes themselves.
-    uint32_t cand0 = 0, cand1 = 0, cand2 = 0, a_last = 0;
+    // landed: they all lie in the last aligned dword of a.  The same holds for b with n % 4 != 0.
+    // The three candidates (byte offsets end-3 .. end-1) are worked out once, here, where registers are
+    // plentiful, and kept in scalar registers.
+    const bool a_tail = TAILS && (p.lda & 3) != 0 && p.k > 0;
+    const bool b_tail = TAILS && MODE != 2 && (p.n & 3) != 0 && p.k > 0;
+    uint32_t acand0 = 0, acand1 = 0, acand2 = 0, a_last = 0, bcand0 = 0, bcand1 = 0, bcand2 = 0, b_last = 0;
     if (a_tail) {
-        auto candidate = [&](uint32_t o) __attribute__((always_inline)) -> uint32_t {
-            const uint32_t krow = o / (uint32_t)p.lda, row = o - krow * (uint32_t)p.lda;
-            const bool lost = krow * (uint32_t)p.lda + (row & ~3u) + 4u > a_end;          // its dword crosses the end
-            return lost ? (0x80000000u | ((krow - ((uint32_t)p.k - 3u)) << 29) | row) : 0u;
-        };
-        cand0 = candidate(a_end - 3); cand1 = candidate(a_end - 2); cand2 = candidate(a_end - 1);
-        a_last = *(const uint32_t*)(p.a + (a_end - 4));
+        const uint32_t end = (uint32_t)p.k * (uint32_t)p.lda;
+        acand0 = tail_candidate(end - 3, (uint32_t)p.lda, end, (uint32_t)p.k);
+        acand1 = tail_candidate(end - 2, (uint32_t)p.lda, end, (uint32_t)p.k);
+        acand2 = tail_candidate(end - 1, (uint32_t)p.lda, end, (uint32_t)p.k);
+        a_last = *(const uint32_t*)(p.a + (end - 4));
     }
-    // (the load is consumed here, not inside the K loop)
-    cand0 = __builtin_amdgcn_readfirstlane(cand0); cand1 = __builtin_amdgcn_readfirstlane(cand1);
-    cand2 = __builtin_amdgcn_readfirstlane(cand2); a_last = __builtin_amdgcn_readfirstlane(a_last);
+    if (b_tail) {
+        const uint32_t end = (uint32_t)p.k * (uint32_t)p.n;
+        bcand0 = tail_candidate(end - 3, (uint32_t)p.n, end, (uint32_t)p.k);
+        bcand1 = tail_candidate(end - 2, (uint32_t)p.n, end, (uint32_t)p.k);
+        bcand2 = tail_candidate(end - 1, (uint32_t)p.n, end, (uint32_t)p.k);
+        b_last = *(const uint32_t*)(p.b + (end - 4));
+    }
+    // (the loads are consumed here, not inside the K loop)
+    acand0 = __builtin_amdgcn_readfirstlane(acand0); acand1 = __builtin_amdgcn_readfirstlane(acand1);
+    acand2 = __builtin_amdgcn_readfirstlane(acand2); a_last = __builtin_amdgcn_readfirstlane(a_last);
+    bcand0 = __builtin_amdgcn_readfirstlane(bcand0); bcand1 = __builtin_amdgcn_readfirstlane(bcand1);
+    bcand2 = __builtin_amdgcn_readfirstlane(bcand2); b_last = __builtin_amdgcn_readfirstlane(b_last);
+    // stage: the tile's last K block; called by every wave right behind the barrier that publishes that
+    // block; ends with a second barrier
+#define FP8BS_PATCH_TAILS(stage, spare_stage)                                                                                              \
+    do {                                                                                                                                   \
+        patch_tail_bytes<BM, C::CPR_A>(lds + (stage) * C::STAGE_BYTES, lds + (spare_stage) * C::STAGE_BYTES + C::STAGE_BYTES - 1,          \
+                                       patch_tile && a_tail, m0, acand0, acand1, acand2, a_last, tid);                                     \
+        patch_tail_bytes<BN, C::CPR_B>(lds + (stage) * C::STAGE_BYTES + C::A_BYTES, lds + (spare_stage) * C::STAGE_BYTES + C::STAGE_BYTES - 1, \
+                                       patch_tile && b_tail, n0, bcand0, bcand1, bcand2, b_last, tid);                                     \
+        __syncthreads();                                                                                                                   \
+    } while (0)
+
     Tile cur = pick_tile(0);
     if (!cur.valid) return;
     CopyPlan cp = copy_plan(cur);
@@ -482,7 +506,7 @@ void gemm_tr_kernel(const GemmArgs p) {
         for (int u = 0; u < C::NT; u++) acc[t][u] = (v4f){0.f, 0.f, 0.f, 0.f};
 
     const int nkb = kb_end - kb_begin;
-    const bool patch_tile = a_tail && kb_end * KBLK == p.k;       // this tile's last K block is the last of a
+    const bool patch_tile = TAILS && kb_end * KBLK == p.k;        // this tile's last K block is the last of a and b
     if (nkb > 0) {
         constexpr int STEPS = C::MT * C::NT;
         constexpr int LAG = 3, RING = 4;      // fold the result of step s-LAG while step s runs
@@ -515,7 +539,7 @@ void gemm_tr_kernel(const GemmArgs p) {
             else { if (sb) wait_vmcnt<EPI_STORES>(); else wait_vmcnt<0>(); }
         }
         __syncthreads();
-        if (ATAIL && nkb == 1) patch_a_tail<BM, C::CPR_A>(lds, lds + C::STAGE_BYTES - 1, patch_tile, m0, cand0, cand1, cand2, a_last, tid);
+        if (TAILS && nkb == 1) FP8BS_PATCH_TAILS(0, 1);
         if (nkb > NSTAGE - 1) {
             [&]<int... Q>(std::integer_sequence<int, Q...>) {
                 (issue_one(cp, NSTAGE - 1, NSTAGE - 1, std::integral_constant<int, Q>{}), ...);
@@ -563,7 +587,7 @@ void gemm_tr_kernel(const GemmArgs p) {
                 }
                 wait_next_block();
                 __syncthreads();
-                if constexpr (ATAIL && LANDS_LAST) patch_a_tail<BM, C::CPR_A>(lds + next_stage * C::STAGE_BYTES, lds + cur_stage * C::STAGE_BYTES + C::STAGE_BYTES - 1, patch_tile, m0, cand0, cand1, cand2, a_last, tid);
+                if constexpr (TAILS && LANDS_LAST) FP8BS_PATCH_TAILS(next_stage, cur_stage);
                 if constexpr (HAS_LATE) {
                     [&]<int... Q>(std::integer_sequence<int, Q...>) {
                         (issue_one(cp, cur_stage, j + NSTAGE, std::integral_constant<int, Q>{}), ...);
@@ -596,7 +620,7 @@ void gemm_tr_kernel(const GemmArgs p) {
                         // block is complete in the other stage and this stage may be overwritten.
                         wait_next_block();
                         __syncthreads();
-                        if constexpr (ATAIL && LANDS_LAST) patch_a_tail<BM, C::CPR_A>(lds + next_stage * C::STAGE_BYTES, lds + cur_stage * C::STAGE_BYTES + C::STAGE_BYTES - 1, patch_tile, m0, cand0, cand1, cand2, a_last, tid);
+                        if constexpr (TAILS && LANDS_LAST) FP8BS_PATCH_TAILS(next_stage, cur_stage);
                     }
                     const v4f z = {0.f, 0.f, 0.f, 0.f};
                     ring[s % RING] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(breg[u & 1], areg[t], z, 0, 0, 0, 0, 0, 0);
@@ -746,15 +770,36 @@ void gemm_tr_kernel(const GemmArgs p) {
                 const int row = m0 + wave_row0 + pass_row0 + lane_r;
                 const bool ok = col_ok && row >= row_lo && row < row_hi;
                 __amdgpu_buffer_rsrc_t c_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(c_tile + (size_t)pass_row0 * ldc), 0, 0xFFFFFFF0u, 0x00020000);
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, val), c_rsrc, ok ? lane_off : 0xFFFFFFFFu, 0, 2);   // nontemporal: written once, not read again here
+                if constexpr (!TAILS) {
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, val), c_rsrc, ok ? lane_off : 0xFFFFFFFFu, 0, 2);   // nontemporal: written once, not read again here
+                } else {
+                    // n not a multiple of eight: the chunk that holds a row's last columns is stored in
+                    // pieces of 4, 2 and 1 elements (the bits of the number of columns left), every piece
+                    // its own instruction that the other lanes sit out; rows then start on 2-, 4- or
+                    // 8-byte boundaries only, which the stores take in their stride
+                    int left = ldc - (col0 + wave_col0 + lane_chunk * 8);                  // columns from this chunk's first to the row's end
+                    left = left < 0 ? 0 : (left > 8 ? 8 : left);
+                    const bool part = ok && left < 8;
+                    const v4u v = __builtin_bit_cast(v4u, val);
+                    __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, ok && left == 8 ? lane_off : 0xFFFFFFFFu, 0, 2);
+                    const v2i lo = {val[0], val[1]};
+                    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, lo), c_rsrc, part && (left & 4) ? lane_off : 0xFFFFFFFFu, 0, 2);
+                    const uint32_t d2 = (left & 4) ? v[2] : v[0];                          // elements (left & 4), +1
+                    __builtin_amdgcn_raw_buffer_store_b32(d2, c_rsrc, part && (left & 2) ? lane_off + (uint32_t)(left & 4) * 2u : 0xFFFFFFFFu, 0, 2);
+                    const int e1 = left & 6;                                               // element (left & 6)
+                    const uint32_t d1 = e1 == 0 ? v[0] : e1 == 2 ? v[1] : e1 == 4 ? v[2] : v[3];
+                    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(d1 & 0xFFFFu), c_rsrc, part && (left & 1) ? lane_off + (uint32_t)e1 * 2u : 0xFFFFFFFFu, 0, 2);
+                }
             }
         }
     }
     if (!nxt.valid) break;
-    stores_behind = prefetched && wave_active && MODE != 1;
+    stores_behind = prefetched && wave_active && MODE != 1 && !TAILS;   // (with TAILS the store count is four times EPI_STORES: plain wait)
     cur = nxt; cp = ncp;
     }   // tiles
 }
+
+#undef FP8BS_PATCH_TAILS
 
 // ---------------------------------------------------------------------------------------------------
 // Skinny-M streaming kernel (bandwidth-bound shapes: a few rows of A against a long B).
@@ -1060,11 +1105,12 @@ void gemm_generic_kernel(const GemmArgs p) {
 template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0, int NSTAGE = 2>
 static hipError_t launch_tr(const GemmArgs& a, dim3 grid, hipStream_t stream) {
     using C = TileCfg<BM, BN, WM, WN, MODE, NSTAGE>;
-    // rows of a that are not a multiple of four: the instantiation that repairs the last bytes of a
-    const bool atail = (a.lda & 3) != 0;
-    void (*kern)(const GemmArgs) = atail ? gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI, NSTAGE, true> : gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI, NSTAGE, false>;
+    // rows of a that are not a multiple of four, columns that are not a multiple of eight: the
+    // instantiation that repairs the last bytes of a and b and stores partial chunks of c
+    const bool tails = (a.lda & 3) != 0 || (a.n & 7) != 0;
+    void (*kern)(const GemmArgs) = tails ? gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI, NSTAGE, true> : gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI, NSTAGE, false>;
     static int raised[2][MAX_DEVICES];
-    hipError_t e = raise_lds_limit((const void*)kern, C::LDS_BYTES, raised[atail ? 1 : 0]);
+    hipError_t e = raise_lds_limit((const void*)kern, C::LDS_BYTES, raised[tails ? 1 : 0]);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, grid, dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
     return hipGetLastError();

@@ -88,12 +88,13 @@ size_t fp8bs_workspace_bytes(int m, int n, int k);
 /* Dense GEMM. Replaces `fp8_mm(a,b,as,bs,c,c_tmp)`,
  * 1-amd-fp8-mm/amd-fp8-mm-submission.py:514-579. Inputs are never modified (the reference's
  * pre-transpose branch, :570-571, overwrites a and b; this one does not).
- * Alignment: the fast kernels need n a multiple of 8 and a, b, c, ws on 16-byte boundaries (any m: the
- * tiled kernels read a with its true row length and repair its last one to three bytes in LDS; the
- * streaming kernel, planned for at most 64 rows against a very large b, runs on copies of a and a_scale
- * padded to a multiple of four rows at the head of the workspace when m is not one - without enough
- * workspace the tiled kernels run instead);
- * other shapes or pointers run on the element-wise generic kernel (correct, slow).  a_scale and
+ * Alignment: the fast kernels need a, b, c, ws on 16-byte boundaries; other pointers run on the
+ * element-wise generic kernel (correct, slow).  Any m and n: the tiled kernels read a and b with their
+ * true row lengths, repair their last one to three bytes in LDS and, with n not a multiple of 8, store the
+ * last chunk of every row of c in pieces (no K split is planned then); the streaming kernel, planned for
+ * at most 64 rows against a very large b with n a multiple of 8, runs on copies of a and a_scale padded to
+ * a multiple of four rows at the head of the workspace when m is not one - without enough workspace the
+ * tiled kernels run instead.  a_scale and
  * b_scale must be 4-byte aligned, c 2-byte aligned (FP8BS_ERR_BAD_SHAPE otherwise). */
 int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
                void* c, void* ws, size_t ws_bytes, int m, int n, int k, void* stream);

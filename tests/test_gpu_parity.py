@@ -81,24 +81,25 @@ def test_every_variant_and_split_on_config1(pkg, oracle, dev, variant, split_k):
                                    (132, 200, 256), (20, 24, 128), (516, 264, 384), (268, 2104, 256),
                                    (4095, 512, 256), (1021, 264, 384), (131, 1024, 512), (61, 2048, 1024), (5, 16, 128),
                                    (1, 2048, 1024), (2, 264, 384), (3, 18432, 512), (5, 18432, 512), (1030, 264, 256), (2050, 136, 384),
-                                   (1023, 8, 128), (67, 2112, 640), (7, 64, 128), (2, 8, 256), (255, 256, 128), (257, 192, 384), (513, 136, 1024)])
+                                   (1023, 8, 128), (67, 2112, 640), (7, 64, 128), (2, 8, 256), (255, 256, 128), (257, 192, 384), (513, 136, 1024),
+                                   (128, 190, 256), (256, 257, 128), (64, 1, 128), (100, 50257 // 16, 256), (129, 255, 384), (260, 2108, 256),
+                                   (300, 1001, 128), (512, 4100, 256), (16, 12, 128), (255, 383, 256), (31, 2047, 512)])
 def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
     """N tails (2112 = 16*128 + 64), tiles larger than the matrix, rows and columns that end inside a
-    16-byte chunk (m % 4 == 0, n % 8 == 0: still the vector kernels), shapes only the generic kernel takes."""
+    16-byte chunk, row counts off the 4-row grid and column counts off the 8-column grid."""
     cfg = pkg.inputs.CONFIGS[2]                                   # outlier activations, small weights
     cpu = pkg.inputs.make_dense(cfg, m=m, n=n, k=k)
     out = pkg.custom_kernel(_to(cpu, dev))
     _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d" % (m, n, k))
-    if n % 8 == 0:
-        assert pkg.plan(m, n, k).variant != 1                   # any m: the vector kernels, in two launches if m % 4 != 0
-    if n % 8 == 0:
-        # every tile takes any m (the last bytes of a are repaired in LDS); the streaming kernels m % 4 == 0
-        for variant in (2, 3, 4, 5, 9, 10) + ((6, 7, 8) if m % 4 == 0 else ()):
-            out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1)
-            _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d" % (m, n, k, variant))
-        if k >= 512:
-            out = pkg.custom_kernel(_to(cpu, dev), variant=4, split_k=2)        # the repair happens in the last split only
-            _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant 4 split 2" % (m, n, k))
+    assert pkg.plan(m, n, k).variant != 1                       # any m and n: the vector kernels
+    # every tile takes any m and n (the last bytes of a and b are repaired in LDS, a row's last chunk of
+    # c is stored in pieces); the streaming kernels m % 4 == 0 and n % 8 == 0
+    for variant in (2, 3, 4, 5, 9, 10) + ((6, 7, 8) if m % 4 == 0 and n % 8 == 0 else ()):
+        out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1)
+        _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d" % (m, n, k, variant))
+    if k >= 512 and n % 8 == 0:
+        out = pkg.custom_kernel(_to(cpu, dev), variant=4, split_k=2)        # the repair happens in the last split only
+        _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant 4 split 2" % (m, n, k))
 
 
 @pytest.mark.parametrize("m,n,k,variant", [(8192, 8192, 256, 2), (8188, 4104, 128, 0), (4096, 8192, 384, 5),
@@ -226,6 +227,24 @@ def test_rows_not_a_multiple_of_four_without_a_workspace(pkg, oracle, dev, m, n,
     _check(oracle, c, oracle.ref_kernel(cpu), "no workspace %dx%dx%d" % (m, n, k))
     with_ws = pkg.custom_kernel((a, b, a_scale, b_scale, torch.full_like(c, float("nan"))))
     _check(oracle, with_ws, oracle.ref_kernel(cpu), "workspace %dx%dx%d" % (m, n, k))
+
+
+@pytest.mark.parametrize("m,n,k,variant", [(130, 190, 256, 0), (64, 1001, 128, 2), (33, 257, 128, 4), (260, 2111, 256, 9), (129, 127, 384, 10), (5, 3, 128, 3)])
+def test_nothing_is_written_outside_c(pkg, oracle, dev, m, n, k, variant):
+    """c sits in the middle of a larger buffer of a sentinel value: with rows that end inside a 16-byte chunk
+    the kernels store the last chunk of a row in pieces, and neither the bytes in front of c nor those behind
+    its last row may change.  Every row is also checked against the oracle (a piece stored one row too far
+    would land on the next row's first columns)."""
+    cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[2], m=m, n=n, k=k)
+    a, b, a_scale, b_scale, _ = _to(cpu, dev)
+    pad = 64                                                  # elements in front (keeps c on a 16-byte boundary) and behind
+    buf = torch.full((pad + m * n + pad,), -7.0, dtype=torch.bfloat16, device=dev)
+    c = buf[pad:pad + m * n].view(m, n)
+    assert c.data_ptr() % 16 == 0
+    out = pkg.custom_kernel((a, b, a_scale, b_scale, c), variant=variant, split_k=1 if variant else 0)
+    torch.cuda.synchronize()
+    assert bool((buf[:pad] == -7.0).all()) and bool((buf[pad + m * n:] == -7.0).all()), "bytes outside c were written"
+    _check(oracle, out, oracle.ref_kernel(cpu), "sentinel %dx%dx%d variant %d" % (m, n, k, variant))
 
 
 def test_empty_shapes(pkg, dev):
