@@ -59,15 +59,10 @@ void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out)
     out->workspace_bytes = split_k > 1 ? (uint64_t)split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
 }
 
-// The streaming kernels copy a in dwords that must not cross the end of its buffer: they need m % 4 == 0.
-// For other m, a and a_scale are first copied into matrices of mp = m rounded up to four rows at the head
-// of the workspace (k * mp bytes: the streaming kernels only ever see a few rows).
-uint64_t pad_bytes(int k, int mp) { return (((uint64_t)k * (uint64_t)mp + (uint64_t)(k / KBLK) * (uint64_t)mp * 4u) + 255u) & ~(uint64_t)255u; }
-
 // Rows of c (n bf16) that keep 16-byte stores aligned: what the streaming kernels, the K split (its
 // reduction works on groups of eight outputs), the grouped walk and the fused epilogue need.  The tiled
 // kernels without a K split take any m and n (they repair the last bytes of a and b themselves and store
-// a row's last chunk of c in pieces); the streaming kernels also need m % 4 == 0.
+// a row's last chunk of c in pieces); the streaming kernels take any m.
 bool vector_shape(int n) { return (n % 8) == 0; }
 
 // The streaming kernel is kept for what it was built for: at most 64 rows against a B too large for the
@@ -120,7 +115,7 @@ void choose_tiled(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     fill_plan(m, n, k, best_variant, best_split, out);
 }
 
-// The streaming kernel with the K split that fills the CUs (m a multiple of four).
+// The streaming kernel with the K split that fills the CUs.
 void choose_streaming(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     if (num_cus <= 0) num_cus = 256;
     int kbt = k / KBLK;
@@ -137,16 +132,11 @@ void choose_streaming(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     fill_plan(m, n, k, FP8BS_VARIANT_SKINNY64x144, best_s, out);
 }
 
-// Shape-family rule.  A few rows against a very large B -> the streaming kernel (on padded copies of
-// a / a_scale if m % 4 != 0).  Everything else -> the tiled kernel.
+// Shape-family rule.  A few rows against a very large B -> the streaming kernel.  Everything else -> the
+// tiled kernel.
 void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
-    if (vector_shape(n) && streaming_shape(m, n, k)) {
-        const int mp = (m + 3) & ~3;
-        choose_streaming(mp, n, k, num_cus, out);
-        if (mp != m) out->workspace_bytes += pad_bytes(k, mp);
-    } else {
-        choose_tiled(m, n, k, num_cus, out);
-    }
+    if (vector_shape(n) && streaming_shape(m, n, k)) choose_streaming(m, n, k, num_cus, out);
+    else choose_tiled(m, n, k, num_cus, out);
 }
 
 bool is_streaming_variant(int v) { return v == FP8BS_VARIANT_SKINNY64x144 || v == FP8BS_VARIANT_SKINNY64x256 || v == FP8BS_VARIANT_SKINNY64x288; }
@@ -216,37 +206,23 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
         if (variant != FP8BS_VARIANT_AUTO && variant != FP8BS_VARIANT_GENERIC) return FP8BS_ERR_BAD_VARIANT;
         variant = FP8BS_VARIANT_GENERIC;
     }
-    bool padded = false;        // the streaming kernel runs on padded copies of a / a_scale in the workspace
     if (variant == FP8BS_VARIANT_AUTO) {
         choose(m, n, k, 0, &plan);
-        if (is_streaming_variant(plan.variant) && (m % 4) != 0) {
-            const uint64_t planes = plan.split_k > 1 ? (uint64_t)plan.split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
-            if (split_k == 0 && ws && ws_bytes >= pad_bytes(k, (m + 3) & ~3) + planes) padded = true;
-            else choose_tiled(m, n, k, 0, &plan);     // no room for the copies (or a forced split): the tiled kernels take any m
-        }
         if (split_k > 1 && !vector_shape(n)) return FP8BS_ERR_BAD_VARIANT;
         if (split_k > 0) fill_plan(m, n, k, plan.variant, split_k, &plan);
     } else {
         VariantInfo vi{};
         if (!variant_info(variant, &vi)) return FP8BS_ERR_BAD_VARIANT;
         if (variant != FP8BS_VARIANT_GENERIC && !vector_shape(n) && (is_streaming_variant(variant) || split_k > 1)) return FP8BS_ERR_BAD_VARIANT;
-        if (is_streaming_variant(variant) && (m % 4) != 0) return FP8BS_ERR_BAD_VARIANT;
+        if (is_streaming_variant(variant) && variant != FP8BS_VARIANT_SKINNY64x144 && (m % 4) != 0) return FP8BS_ERR_BAD_VARIANT;   // only the planner's width repairs a
         fill_plan(m, n, k, variant, split_k > 0 ? split_k : 1, &plan);
     }
-    const int mp = (m + 3) & ~3;
-    const uint64_t pad = padded ? pad_bytes(k, mp) : 0u;
-    if (plan.split_k > 1 && (!ws || ws_bytes < pad + (uint64_t)plan.split_k * (uint64_t)m * (uint64_t)n * 4u)) return FP8BS_ERR_WORKSPACE;
+    if (plan.split_k > 1 && (!ws || ws_bytes < (uint64_t)plan.split_k * (uint64_t)m * (uint64_t)n * 4u)) return FP8BS_ERR_WORKSPACE;
 
     fp8bs::GemmArgs g{};
     g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.as = a_scale; g.bs = b_scale;
     g.c = (uint16_t*)c; g.ws = (float*)ws; g.row_offsets = nullptr;
     g.m = m; g.n = n; g.k = k; g.lda = m; g.nb = (n + 127) / 128;
-    if (padded) {
-        uint8_t* ap = (uint8_t*)ws;
-        float* asp = (float*)(ap + (size_t)k * mp);
-        if (fp8bs::launch_pad_rows((const uint8_t*)a, a_scale, ap, asp, m, mp, k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
-        g.a = ap; g.as = asp; g.lda = mp; g.ws = (float*)((uint8_t*)ws + pad);
-    }
     g.split_k = plan.split_k;
     g.kb_per_split = (int)cdiv(k / KBLK, plan.split_k);
     g.band_h = 4;

@@ -17,7 +17,7 @@ struct GemmArgs {
     float* ws;              // split-K partial planes [split_k][m][n]
     const int32_t* row_offsets;
     int m, n, k;
-    int lda;                // bytes per k row of a (the row count of the whole matrix; the streaming kernels need a multiple of 4)
+    int lda;                // bytes per k row of a (the row count of the whole matrix)
     int nb;                 // ceil(n / 128)
     int split_k, kb_per_split;
     int band_h;             // tile rows per band of the tile walk
@@ -45,7 +45,6 @@ inline hipError_t raise_lds_limit(const void* kernel, int bytes, int* raised) {
 // mode: 0 dense bf16, 1 dense split-K partials, 2 grouped.  variant: FP8BS_VARIANT_* (not AUTO).
 hipError_t launch_gemm(int variant, int mode, const GemmArgs& args, hipStream_t stream);
 hipError_t launch_splitk_reduce(const float* ws, uint16_t* c, size_t mn, int split_k, hipStream_t stream);
-hipError_t launch_pad_rows(const uint8_t* a, const float* as, uint8_t* ap, float* asp, int m, int mp, int k, hipStream_t stream);
 int variant_lds_bytes(int variant);
 
 }  // namespace fp8bs

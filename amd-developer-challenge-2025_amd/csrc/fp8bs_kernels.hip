@@ -845,7 +845,8 @@ struct SkinnyCfg {
 // MTV: the 16-row m tiles that get multiplied, 1..4.  Fewer than 4 only when the whole matrix has at
 // most 16*MTV rows (a decode step has one to a few): a compile-time count, because a run-time test per
 // m tile put branches between the MFMAs and their folds, and results read back too early were seen.
-template <int BN_, int NSTAGE_, int MODE, int MTV>
+// TAILS: lda is not a multiple of four; the last bytes of a are repaired in LDS as in the tiled kernel.
+template <int BN_, int NSTAGE_, int MODE, int MTV, bool TAILS = false>
 __global__ __launch_bounds__(256)
 void gemm_skinny_kernel(const GemmArgs p) {
     using C = SkinnyCfg<BN_, NSTAGE_>;
@@ -940,6 +941,19 @@ void gemm_skinny_kernel(const GemmArgs p) {
 #pragma unroll
         for (int x = 0; x < C::NT_MAX; x++) acc[t][x] = (v4f){0.f, 0.f, 0.f, 0.f};
 
+    // rows of a that are not a multiple of four: see the tiled kernel
+    const bool a_tail = TAILS && (p.lda & 3) != 0 && p.k > 0 && kb_end == kbt && nkb > 0;
+    uint32_t acand0 = 0, acand1 = 0, acand2 = 0, a_last = 0;
+    if (a_tail) {
+        const uint32_t end = (uint32_t)p.k * (uint32_t)p.lda;
+        acand0 = tail_candidate(end - 3, (uint32_t)p.lda, end, (uint32_t)p.k);
+        acand1 = tail_candidate(end - 2, (uint32_t)p.lda, end, (uint32_t)p.k);
+        acand2 = tail_candidate(end - 1, (uint32_t)p.lda, end, (uint32_t)p.k);
+        a_last = *(const uint32_t*)(p.a + (end - 4));
+    }
+    acand0 = __builtin_amdgcn_readfirstlane(acand0); acand1 = __builtin_amdgcn_readfirstlane(acand1);
+    acand2 = __builtin_amdgcn_readfirstlane(acand2); a_last = __builtin_amdgcn_readfirstlane(a_last);
+
     // The loop is instantiated once per wave index: which copies a wave issues and which n tiles it
     // multiplies then are compile-time facts, and the loop body has no branches.
     auto k_loop = [&](auto wave_tag) {
@@ -951,6 +965,13 @@ void gemm_skinny_kernel(const GemmArgs p) {
         // the NSTAGE-2 blocks issued after block j may still be on their way
         wait_vmcnt<(C::NSTAGE - 2) * C::COPIES>();
         __syncthreads();      // block j complete in LDS; everyone is done with the stage of block j-1
+        if constexpr (TAILS) {
+            if (j == nkb - 1) {   // the last block of a has landed: its last bytes, then a second barrier
+                unsigned char* st = lds + (j % C::NSTAGE) * C::STAGE_BYTES;
+                patch_tail_bytes<C::BM, C::CPR_A>(st, st + C::STAGE_BYTES - 1, a_tail, m0, acand0, acand1, acand2, a_last, tid);
+                __syncthreads();
+            }
+        }
         issue_block(wave_tag, j + C::NSTAGE - 1);
 
         const unsigned char* sbase = lds + (j % C::NSTAGE) * C::STAGE_BYTES;
@@ -1159,30 +1180,30 @@ static hipError_t launch_shape(const GemmArgs& a, int mode, hipStream_t stream) 
     return launch_tr<BM, BN, WM, WN, 0, 0, NSTAGE>(a, grid, stream);
 }
 
+template <int BN, int NSTAGE, int MODE, bool TAILS>
+static void (*skinny_kernel_for(int mtv))(const GemmArgs) {
+    if constexpr (BN == 144) {
+        if (mtv == 1) return gemm_skinny_kernel<BN, NSTAGE, MODE, 1, TAILS>;
+        if (mtv == 2) return gemm_skinny_kernel<BN, NSTAGE, MODE, 2, TAILS>;
+        if (mtv == 3) return gemm_skinny_kernel<BN, NSTAGE, MODE, 3, TAILS>;
+    }
+    return gemm_skinny_kernel<BN, NSTAGE, MODE, 4, TAILS>;
+}
+
 template <int BN, int NSTAGE>
 static hipError_t launch_skinny(const GemmArgs& a, int mode, hipStream_t stream) {
     if (mode == 2 || a.epi != 0) return hipErrorInvalidValue;
     using C = SkinnyCfg<BN, NSTAGE>;
     // m tiles with rows: fewer than 4 only for the planner's tile width and a matrix of at most 48 rows
     const int mtv = (BN == 144 && a.m <= 48) ? (a.m + 15) / 16 : 4;
-    void (*kern)(const GemmArgs) = nullptr;
-    if (mode == 1) {
-        kern = gemm_skinny_kernel<BN, NSTAGE, 1, 4>;
-        if constexpr (BN == 144) {
-            if (mtv == 1) kern = gemm_skinny_kernel<BN, NSTAGE, 1, 1>;
-            if (mtv == 2) kern = gemm_skinny_kernel<BN, NSTAGE, 1, 2>;
-            if (mtv == 3) kern = gemm_skinny_kernel<BN, NSTAGE, 1, 3>;
-        }
-    } else {
-        kern = gemm_skinny_kernel<BN, NSTAGE, 0, 4>;
-        if constexpr (BN == 144) {
-            if (mtv == 1) kern = gemm_skinny_kernel<BN, NSTAGE, 0, 1>;
-            if (mtv == 2) kern = gemm_skinny_kernel<BN, NSTAGE, 0, 2>;
-            if (mtv == 3) kern = gemm_skinny_kernel<BN, NSTAGE, 0, 3>;
-        }
+    const bool tails = (a.lda & 3) != 0;      // the instantiation that repairs the last bytes of a: planner's tile width only
+    void (*kern)(const GemmArgs) = mode == 1 ? skinny_kernel_for<BN, NSTAGE, 1, false>(mtv) : skinny_kernel_for<BN, NSTAGE, 0, false>(mtv);
+    if (tails) {
+        if constexpr (BN == 144) kern = mode == 1 ? skinny_kernel_for<BN, NSTAGE, 1, true>(mtv) : skinny_kernel_for<BN, NSTAGE, 0, true>(mtv);
+        else return hipErrorInvalidValue;
     }
-    static int raised[8][MAX_DEVICES];
-    hipError_t e = raise_lds_limit((const void*)kern, C::LDS_BYTES, raised[(mode == 1 ? 4 : 0) + mtv - 1]);
+    static int raised[16][MAX_DEVICES];
+    hipError_t e = raise_lds_limit((const void*)kern, C::LDS_BYTES, raised[(tails ? 8 : 0) + (mode == 1 ? 4 : 0) + mtv - 1]);
     if (e != hipSuccess) return e;
     int tiles = ((a.n + C::BN - 1) / C::BN) * a.split_k * ((a.m + C::BM - 1) / C::BM);
     hipLaunchKernelGGL(kern, dim3(tiles), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
@@ -1207,34 +1228,6 @@ hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t str
         case 10: return launch_shape<256, 128, 64, 64, false, 3>(a, mode, stream);
         default: return hipErrorInvalidValue;
     }
-}
-
-// A number of rows that is not a multiple of four (a few tokens of a decode step, an odd batch): copy a
-// and a_scale into matrices of mp = m rounded up to four rows (the added rows are zero).  With k rows of
-// mp bytes every 4-byte load of the vector kernels stays on a dword of its own and inside the buffer.
-__global__ __launch_bounds__(256)
-void pad_rows_kernel(const uint8_t* __restrict__ a, const float* __restrict__ as, uint8_t* __restrict__ ap, float* __restrict__ asp, int m, int mp, int k) {
-    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    const int groups = mp / 4;
-    if (idx < (size_t)k * groups) {
-        const size_t kk = idx / groups;
-        const int r0 = 4 * (int)(idx % groups);
-        uint32_t w = 0;
-        for (int i = 0; i < 4; i++)
-            if (r0 + i < m) w |= (uint32_t)a[kk * m + r0 + i] << (8 * i);
-        *(uint32_t*)(ap + 4 * idx) = w;
-    }
-    if (idx < (size_t)(k / KBLK) * mp) {
-        const size_t kb = idx / mp;
-        const int r = (int)(idx % mp);
-        asp[idx] = r < m ? as[kb * m + r] : 0.f;
-    }
-}
-
-hipError_t launch_pad_rows(const uint8_t* a, const float* as, uint8_t* ap, float* asp, int m, int mp, int k, hipStream_t stream) {
-    const size_t threads = (size_t)k * (mp / 4);                  // more than the (k/128)*mp scale entries
-    hipLaunchKernelGGL(pad_rows_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, a, as, ap, asp, m, mp, k);
-    return hipGetLastError();
 }
 
 hipError_t launch_splitk_reduce(const float* ws, uint16_t* c, size_t mn, int split_k, hipStream_t stream) {

@@ -198,7 +198,7 @@ def main():
         us, us_min = time_calls(lambda i: pkg.custom_kernel(sets[i % nsets]), args.steps, args.warmup)
         per_config[dcfg.name] = {"us": round(us, 2), "us_min": round(us_min, 2), "gbs": round(by / us * 1e-3, 1), "bytes": by,
                                  "input_sets": nsets, "bound": "hbm", "frac": round(by / us * 1e-3 / PEAK_HBM_GBS, 4),
-                                 "note": "one row: a and a_scale copied to four-row matrices, then the streaming kernel"}
+                                 "note": "one row: the streaming kernel with a K split of 2, then the reduction"}
         sets = None
     # ---- the quantisers in front of the GEMM (HBM-bound): activations of configuration 3, one expert's
     # weights of configuration 5; 4 rotating inputs (> 256 MB in total) so that reads come from HBM ----

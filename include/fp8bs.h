@@ -92,9 +92,7 @@ size_t fp8bs_workspace_bytes(int m, int n, int k);
  * element-wise generic kernel (correct, slow).  Any m and n: the tiled kernels read a and b with their
  * true row lengths, repair their last one to three bytes in LDS and, with n not a multiple of 8, store the
  * last chunk of every row of c in pieces (no K split is planned then); the streaming kernel, planned for
- * at most 64 rows against a very large b with n a multiple of 8, runs on copies of a and a_scale padded to
- * a multiple of four rows at the head of the workspace when m is not one - without enough workspace the
- * tiled kernels run instead.  a_scale and
+ * at most 64 rows against a very large b with n a multiple of 8, repairs a the same way.  a_scale and
  * b_scale must be 4-byte aligned, c 2-byte aligned (FP8BS_ERR_BAD_SHAPE otherwise). */
 int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
                void* c, void* ws, size_t ws_bytes, int m, int n, int k, void* stream);

@@ -93,13 +93,14 @@ def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
     _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d" % (m, n, k))
     assert pkg.plan(m, n, k).variant != 1                       # any m and n: the vector kernels
     # every tile takes any m and n (the last bytes of a and b are repaired in LDS, a row's last chunk of
-    # c is stored in pieces); the streaming kernels m % 4 == 0 and n % 8 == 0
-    for variant in (2, 3, 4, 5, 9, 10) + ((6, 7, 8) if m % 4 == 0 and n % 8 == 0 else ()):
+    # c is stored in pieces); the streaming kernels n % 8 == 0, and all but the planner's width m % 4 == 0
+    for variant in (2, 3, 4, 5, 9, 10) + ((6,) if n % 8 == 0 else ()) + ((7, 8) if m % 4 == 0 and n % 8 == 0 else ()):
         out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1)
         _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d" % (m, n, k, variant))
     if k >= 512 and n % 8 == 0:
-        out = pkg.custom_kernel(_to(cpu, dev), variant=4, split_k=2)        # the repair happens in the last split only
-        _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant 4 split 2" % (m, n, k))
+        for variant in (4, 6):
+            out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=2)  # the repair happens in the last split only
+            _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d split 2" % (m, n, k, variant))
 
 
 @pytest.mark.parametrize("m,n,k,variant", [(8192, 8192, 256, 2), (8188, 4104, 128, 0), (4096, 8192, 384, 5),
@@ -245,6 +246,18 @@ def test_nothing_is_written_outside_c(pkg, oracle, dev, m, n, k, variant):
     torch.cuda.synchronize()
     assert bool((buf[:pad] == -7.0).all()) and bool((buf[pad + m * n:] == -7.0).all()), "bytes outside c were written"
     _check(oracle, out, oracle.ref_kernel(cpu), "sentinel %dx%dx%d variant %d" % (m, n, k, variant))
+
+
+@pytest.mark.parametrize("m", [1, 3, 5, 18, 63])
+def test_decode_rows_against_a_large_b(pkg, oracle, dev, m):
+    """A few token rows against configuration 4's weights (132 MB): the streaming kernel with a K split,
+    row counts off the 4-row grid included (one to three rows: k rows of a shorter than a dword)."""
+    cfg = pkg.inputs.CONFIGS[3]
+    cpu = pkg.inputs.make_dense(cfg, m=m)
+    plan = pkg.plan(m, cfg.n, cfg.k)
+    assert plan.variant == 6 and plan.split_k > 1
+    out = pkg.custom_kernel(_to(cpu, dev))
+    _check(oracle, out, oracle.ref_kernel(cpu), "decode %d rows" % m)
 
 
 def test_empty_shapes(pkg, dev):
