@@ -73,8 +73,8 @@ bool vector_shape(int n) { return (n % 8) == 0; }
 bool streaming_shape(int m, int n, int k) { return m <= 64 && (double)n * (double)k >= 96.0e6; }
 
 // The tile shape and K split of the tiled MFMA kernel that finish soonest (any m; any n without a split).
-void choose_tiled(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
-    const bool may_split = vector_shape(n);
+void choose_tiled(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may_split = true) {
+    may_split = may_split && vector_shape(n);
     if (num_cus <= 0) num_cus = 256;
     int kbt = k / KBLK;
     // The tile shape and K split that finish soonest under a cost model in
@@ -153,9 +153,8 @@ int check_common(const void* a, const void* b, const float* as, const float* bs,
     return FP8BS_OK;
 }
 
-// The tiled and streaming kernels copy and store 16 bytes at a time: operands, output and workspace
-// must start on 16-byte boundaries (with vector_shape() the copies then stay dword-aligned and the
-// stores 16-byte aligned).  Anything else is left to the generic kernel, which accesses single elements.
+// Operands and output on 16-byte boundaries: what the streaming kernels, the K split, the grouped walk and
+// the fused epilogue need (aligned 8- and 16-byte stores of c).
 bool vector_aligned(const void* a, const void* b, const void* c, const void* ws) {
     return ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)ws) & 15) == 0);
 }
@@ -202,18 +201,21 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
     hipStream_t s = (hipStream_t)stream;
     fp8bs_plan_t plan{};
     if (k == 0) variant = FP8BS_VARIANT_GENERIC;   // empty sum: the generic kernel writes zeros
-    if (!vector_aligned(a, b, c, ws)) {
-        if (variant != FP8BS_VARIANT_AUTO && variant != FP8BS_VARIANT_GENERIC) return FP8BS_ERR_BAD_VARIANT;
-        variant = FP8BS_VARIANT_GENERIC;
-    }
+    // Operands off the 16-byte grid: the tiled kernels without a K split take them as they take rows of a, b
+    // and c that start anywhere (the same instantiation); the K split's reduction and the streaming
+    // kernels store c in aligned 8- and 16-byte pieces and are left out.  A misaligned workspace is not used.
+    const bool aligned = vector_aligned(a, b, c, nullptr);
+    if (((uintptr_t)ws & 15) != 0) { ws = nullptr; ws_bytes = 0; }
+    const bool simple = aligned && vector_shape(n);      // K split and streaming kernels possible
     if (variant == FP8BS_VARIANT_AUTO) {
-        choose(m, n, k, 0, &plan);
-        if (split_k > 1 && !vector_shape(n)) return FP8BS_ERR_BAD_VARIANT;
+        if (aligned) choose(m, n, k, 0, &plan);
+        else choose_tiled(m, n, k, 0, &plan, false);
+        if (split_k > 1 && !simple) return FP8BS_ERR_BAD_VARIANT;
         if (split_k > 0) fill_plan(m, n, k, plan.variant, split_k, &plan);
     } else {
         VariantInfo vi{};
         if (!variant_info(variant, &vi)) return FP8BS_ERR_BAD_VARIANT;
-        if (variant != FP8BS_VARIANT_GENERIC && !vector_shape(n) && (is_streaming_variant(variant) || split_k > 1)) return FP8BS_ERR_BAD_VARIANT;
+        if (variant != FP8BS_VARIANT_GENERIC && !simple && (is_streaming_variant(variant) || split_k > 1)) return FP8BS_ERR_BAD_VARIANT;
         if (is_streaming_variant(variant) && variant != FP8BS_VARIANT_SKINNY64x144 && (m % 4) != 0) return FP8BS_ERR_BAD_VARIANT;   // only the planner's width repairs a
         fill_plan(m, n, k, variant, split_k > 0 ? split_k : 1, &plan);
     }

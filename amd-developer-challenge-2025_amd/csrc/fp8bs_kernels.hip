@@ -191,6 +191,10 @@ __device__ __forceinline__ void patch_tail_bytes(unsigned char* tile, unsigned c
         *(apply != 0 ? dst : spare) = (unsigned char)(last >> (8 * (c + 1)));
     }
 }
+// The last four bytes of an operand, which may start on any byte.
+__device__ __forceinline__ uint32_t load_last_dword(const uint8_t* q) {
+    return (uint32_t)q[0] | ((uint32_t)q[1] << 8) | ((uint32_t)q[2] << 16) | ((uint32_t)q[3] << 24);
+}
 // The three candidates of an operand whose k rows are ld bytes long and whose buffer ends at `end`.
 __device__ __forceinline__ uint32_t tail_candidate(uint32_t o, uint32_t ld, uint32_t end, uint32_t k) {
     const uint32_t krow = o / ld, x = o - krow * ld;
@@ -456,14 +460,14 @@ void gemm_tr_kernel(const GemmArgs p) {
         acand0 = tail_candidate(end - 3, (uint32_t)p.lda, end, (uint32_t)p.k);
         acand1 = tail_candidate(end - 2, (uint32_t)p.lda, end, (uint32_t)p.k);
         acand2 = tail_candidate(end - 1, (uint32_t)p.lda, end, (uint32_t)p.k);
-        a_last = *(const uint32_t*)(p.a + (end - 4));
+        a_last = load_last_dword(p.a + (end - 4));
     }
     if (b_tail) {
         const uint32_t end = (uint32_t)p.k * (uint32_t)p.n;
         bcand0 = tail_candidate(end - 3, (uint32_t)p.n, end, (uint32_t)p.k);
         bcand1 = tail_candidate(end - 2, (uint32_t)p.n, end, (uint32_t)p.k);
         bcand2 = tail_candidate(end - 1, (uint32_t)p.n, end, (uint32_t)p.k);
-        b_last = *(const uint32_t*)(p.b + (end - 4));
+        b_last = load_last_dword(p.b + (end - 4));
     }
     // (the loads are consumed here, not inside the K loop)
     acand0 = __builtin_amdgcn_readfirstlane(acand0); acand1 = __builtin_amdgcn_readfirstlane(acand1);
@@ -949,7 +953,7 @@ void gemm_skinny_kernel(const GemmArgs p) {
         acand0 = tail_candidate(end - 3, (uint32_t)p.lda, end, (uint32_t)p.k);
         acand1 = tail_candidate(end - 2, (uint32_t)p.lda, end, (uint32_t)p.k);
         acand2 = tail_candidate(end - 1, (uint32_t)p.lda, end, (uint32_t)p.k);
-        a_last = *(const uint32_t*)(p.a + (end - 4));
+        a_last = load_last_dword(p.a + (end - 4));
     }
     acand0 = __builtin_amdgcn_readfirstlane(acand0); acand1 = __builtin_amdgcn_readfirstlane(acand1);
     acand2 = __builtin_amdgcn_readfirstlane(acand2); a_last = __builtin_amdgcn_readfirstlane(a_last);
@@ -1126,9 +1130,10 @@ void gemm_generic_kernel(const GemmArgs p) {
 template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0, int NSTAGE = 2>
 static hipError_t launch_tr(const GemmArgs& a, dim3 grid, hipStream_t stream) {
     using C = TileCfg<BM, BN, WM, WN, MODE, NSTAGE>;
-    // rows of a that are not a multiple of four, columns that are not a multiple of eight: the
-    // instantiation that repairs the last bytes of a and b and stores partial chunks of c
-    const bool tails = (a.lda & 3) != 0 || (a.n & 7) != 0;
+    // rows of a that are not a multiple of four, columns that are not a multiple of eight, operands that
+    // start off the 16-byte grid: the instantiation that repairs the last bytes of a and b and stores c
+    // without assuming any alignment of its rows
+    const bool tails = (a.lda & 3) != 0 || (a.n & 7) != 0 || (((uintptr_t)a.a | (uintptr_t)a.b | (uintptr_t)a.c) & 15) != 0;
     void (*kern)(const GemmArgs) = tails ? gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI, NSTAGE, true> : gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI, NSTAGE, false>;
     static int raised[2][MAX_DEVICES];
     hipError_t e = raise_lds_limit((const void*)kern, C::LDS_BYTES, raised[tails ? 1 : 0]);

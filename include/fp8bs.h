@@ -88,10 +88,10 @@ size_t fp8bs_workspace_bytes(int m, int n, int k);
 /* Dense GEMM. Replaces `fp8_mm(a,b,as,bs,c,c_tmp)`,
  * 1-amd-fp8-mm/amd-fp8-mm-submission.py:514-579. Inputs are never modified (the reference's
  * pre-transpose branch, :570-571, overwrites a and b; this one does not).
- * Alignment: the fast kernels need a, b, c, ws on 16-byte boundaries; other pointers run on the
- * element-wise generic kernel (correct, slow).  Any m and n: the tiled kernels read a and b with their
- * true row lengths, repair their last one to three bytes in LDS and, with n not a multiple of 8, store the
- * last chunk of every row of c in pieces (no K split is planned then); the streaming kernel, planned for
+ * Any m and n, a and b on any byte, c on any bf16 element: the tiled kernels read a and b with their
+ * true row lengths, repair their last one to three bytes in LDS and, with n not a multiple of 8 or c off
+ * the 16-byte grid, store c without assuming any alignment of its rows (no K split is planned then; a
+ * workspace off the 16-byte grid is not used); the streaming kernel, planned for
  * at most 64 rows against a very large b with n a multiple of 8, repairs a the same way.  a_scale and
  * b_scale must be 4-byte aligned, c 2-byte aligned (FP8BS_ERR_BAD_SHAPE otherwise). */
 int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,

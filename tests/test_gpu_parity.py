@@ -194,22 +194,34 @@ def _shifted(t, nbytes):
     return view.t() if rows_major is not t else view
 
 
-@pytest.mark.parametrize("which", ["a", "b", "c"])
-def test_pointers_off_the_16_byte_grid_take_the_generic_kernel(pkg, oracle, dev, which):
-    """The vector kernels need 16-byte aligned operands; anything else must still give the right answer."""
-    cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0], m=64, n=128, k=256)
+@pytest.mark.parametrize("which,shift", [("a", 4), ("a", 1), ("b", 8), ("b", 3), ("c", 2), ("c", 6), ("abc", 5)])
+@pytest.mark.parametrize("m,n,k", [(64, 128, 256), (300, 520, 384), (129, 263, 128)])
+def test_pointers_off_the_16_byte_grid(pkg, oracle, dev, which, shift, m, n, k):
+    """Operands that start anywhere (a, b on any byte, c on any bf16 element): the tiled kernels take them
+    without a K split; the streaming kernels and a forced K split are refused; nothing outside c is written."""
+    cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[2], m=m, n=n, k=k)
     a, b, a_scale, b_scale, c = _to(cpu, dev)
-    if which == "a":
-        a = _shifted(a, 4)
-    elif which == "b":
-        b = _shifted(b, 8)
-    else:
-        c = _shifted(c, 2)
+    if "a" in which:
+        a = _shifted(a, shift)
+    if "b" in which:
+        b = _shifted(b, shift)
+    if "c" in which:
+        buf = torch.full((m * n + 256,), -7.0, dtype=torch.bfloat16, device=dev)
+        off = 64 + (shift & ~1) // 2
+        c = buf[off:off + m * n].view(m, n)
     assert (a.data_ptr() | b.data_ptr() | c.data_ptr()) % 16 != 0
+    ref = oracle.ref_kernel(cpu)
     out = pkg.custom_kernel((a, b, a_scale, b_scale, c))
-    _check(oracle, out, oracle.ref_kernel(cpu), "misaligned " + which)
+    _check(oracle, out, ref, "misaligned %s by %d" % (which, shift))
+    if "c" in which:
+        assert bool((buf[:off] == -7.0).all()) and bool((buf[off + m * n:] == -7.0).all()), "bytes outside c were written"
+    for variant in (2, 4, 9, 10):
+        out = pkg.custom_kernel((a, b, a_scale, b_scale, c), variant=variant, split_k=1)
+        _check(oracle, out, ref, "misaligned %s by %d, variant %d" % (which, shift, variant))
     with pytest.raises(RuntimeError):
-        pkg.custom_kernel((a, b, a_scale, b_scale, c), variant=2, split_k=1)     # a forced vector kernel is refused
+        pkg.custom_kernel((a, b, a_scale, b_scale, c), variant=6, split_k=1)     # the streaming kernels store c in aligned pieces
+    with pytest.raises(RuntimeError):
+        pkg.custom_kernel((a, b, a_scale, b_scale, c), variant=4, split_k=2)     # and so does the reduction of a K split
 
 
 @pytest.mark.parametrize("m,n,k", [(5, 264, 384), (3, 264, 384), (131, 1024, 256), (1027, 136, 256)])
