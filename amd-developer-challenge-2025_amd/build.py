@@ -11,26 +11,44 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 LIB_PATH = os.path.join(HERE, "libfp8bs.so")
-SOURCES = [os.path.join(HERE, "csrc", f) for f in ("fp8bs_kernels.hip", "fp8bs_api.hip", "fp8bs_quant.hip", "fp8bs_route.hip")]
+CSRC = os.path.join(HERE, "csrc")
+SOURCES = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
+OBJ_DIR = os.path.join(HERE, "csrc", "_obj")          # git-ignored build products
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++20", "-shared", "-fPIC",
+    "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC",
     # keep the compiler from forming packed-fp32 VALU instructions
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(HERE, "csrc"),
+    "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
 ]
 
 
-def build(verbose: bool = False) -> str:
-    """Compile the library (always recompiles) and return its path."""
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + ["-o", LIB_PATH] + SOURCES
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if res.returncode != 0:
-        sys.stderr.write(res.stdout)
-        raise RuntimeError("hipcc failed building libfp8bs.so (exit %d)" % res.returncode)
+    return res.returncode, res.stdout
+
+
+def build(verbose: bool = False, jobs: int = 0) -> str:
+    """Compile the library (always recompiles) and return its path.  The tiled kernel is instantiated per
+    tile shape in a translation unit of its own (csrc/fp8bs_tile_*.hip): the files compile side by side."""
+    from concurrent.futures import ThreadPoolExecutor
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    jobs = jobs or min(len(SOURCES), int(os.environ.get("MAX_JOBS", os.cpu_count() or 4)), 16)
+    objs = [os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o") for src in SOURCES]
+    cmds = [[hipcc] + HIPCC_FLAGS + ["-c", "-o", obj, src] for src, obj in zip(SOURCES, objs)]
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        results = list(pool.map(lambda c: _run(c, verbose), cmds))
+    for (rc, out), src in zip(results, SOURCES):
+        if rc != 0:
+            sys.stderr.write(out)
+            raise RuntimeError("hipcc failed compiling %s (exit %d)" % (os.path.basename(src), rc))
+    rc, out = _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs, verbose)
+    if rc != 0:
+        sys.stderr.write(out)
+        raise RuntimeError("hipcc failed linking libfp8bs.so (exit %d)" % rc)
     return LIB_PATH
 
 

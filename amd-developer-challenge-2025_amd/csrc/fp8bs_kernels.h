@@ -44,6 +44,13 @@ inline hipError_t raise_lds_limit(const void* kernel, int bytes, int* raised) {
 
 // mode: 0 dense bf16, 1 dense split-K partials, 2 grouped.  variant: FP8BS_VARIANT_* (not AUTO).
 hipError_t launch_gemm(int variant, int mode, const GemmArgs& args, hipStream_t stream);
+// one per tile shape of the tiled kernel, each in a translation unit of its own
+hipError_t launch_tile_256x256(const GemmArgs& args, int mode, hipStream_t stream);
+hipError_t launch_tile_256x192(const GemmArgs& args, int mode, hipStream_t stream);
+hipError_t launch_tile_256x128(const GemmArgs& args, int mode, hipStream_t stream);
+hipError_t launch_tile_256x128s3(const GemmArgs& args, int mode, hipStream_t stream);
+hipError_t launch_tile_128x128(const GemmArgs& args, int mode, hipStream_t stream);
+hipError_t launch_tile_64x128(const GemmArgs& args, int mode, hipStream_t stream);
 hipError_t launch_splitk_reduce(const float* ws, uint16_t* c, size_t mn, int split_k, hipStream_t stream);
 int variant_lds_bytes(int variant);
 
