@@ -77,7 +77,10 @@ int fp8bs_version(void);
 const char* fp8bs_strerror(int status);
 
 /* Host-only planning: no GPU needed. Replaces the dispatch of
- * 1-amd-fp8-mm/amd-fp8-mm-submission.py:528-578. `num_cus` <= 0 means 256 (MI355X). */
+ * 1-amd-fp8-mm/amd-fp8-mm-submission.py:528-578. `num_cus` <= 0 means 256 (MI355X).  The plan is the one
+ * fp8bs_gemm follows for operands on 16-byte boundaries and a workspace of workspace_bytes; for other
+ * pointers, or without that workspace when split_k > 1, fp8bs_gemm returns FP8BS_ERR_WORKSPACE in the
+ * second case and runs a tiled kernel without a K split in the first. */
 int fp8bs_plan(int m, int n, int k, int num_cus, fp8bs_plan_t* out);
 
 /* Bytes of device workspace fp8bs_gemm needs for this shape (0 when split_k == 1). Replaces the
