@@ -520,7 +520,9 @@ void gemm_tr_kernel(const GemmArgs p) {
         // wave's instruction issue until the texture unit has taken it, and the MFMAs queued behind.
         constexpr int NL_LATE = C::MT < 2 ? C::MT : 2;
         constexpr int NL_EARLY = NLOADS - NL_LATE;
-        constexpr int DMA_EVERY = (STEPS - C::MT) / NL_EARLY >= 2 ? 2 : 1, DMA_FIRST = DMA_EVERY - 1;
+        // (the 192-wide tile is the exception, measured: one copy per step gives it 0.92 us per K block on
+        // one CU against 1.02, while the 256-wide tile loses 4 % that way)
+        constexpr int DMA_EVERY = BN == 192 ? 1 : ((STEPS - C::MT) / NL_EARLY >= 2 ? 2 : 1), DMA_FIRST = DMA_EVERY - 1;
         static_assert(NL_EARLY * DMA_EVERY <= STEPS - C::MT, "not enough steps to issue the copies before the barrier");
 
         // ---- prologue: blocks 0 .. NSTAGE-2 -> stages 0 .. NSTAGE-2 (unless the previous tile already
