@@ -18,7 +18,7 @@ EXPORTS = (
     "fp8bs_gemm_silu_mul", "fp8bs_moe_combine", "fp8bs_convert_fnuz_to_fn",
 )
 
-VARIANT_NAMES = {0: "auto", 1: "generic", 2: "t256x256", 3: "t128x128", 4: "t64x128", 5: "t256x128", 6: "skinny64x144", 7: "skinny64x256", 8: "skinny64x288", 9: "t256x192", 10: "t256x128s3"}
+VARIANT_NAMES = {0: "auto", 1: "generic", 2: "t256x256", 3: "t128x128", 4: "t64x128", 5: "t256x128", 6: "skinny64x144", 7: "skinny64x256", 8: "skinny64x288", 9: "t256x192", 10: "t256x128s3", 11: "t192x192s3"}
 
 
 class Plan(ctypes.Structure):

@@ -370,6 +370,7 @@ hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t str
         case 8: return launch_skinny<288, 3>(a, mode, stream);
         case 9: return launch_tile_256x192(a, mode, stream);
         case 10: return launch_tile_256x128s3(a, mode, stream);
+        case 11: return launch_tile_192x192s3(a, mode, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -392,6 +393,7 @@ int variant_lds_bytes(int variant) {
         case 8: return SkinnyCfg<288, 3>::LDS_BYTES;
         case 9: return TileCfg<256, 192, 64, 96, 0>::LDS_BYTES;
         case 10: return TileCfg<256, 128, 64, 64, 0, 3>::LDS_BYTES;
+        case 11: return TileCfg<192, 192, 48, 96, 0, 3>::LDS_BYTES;
         default: return 0;
     }
 }

@@ -226,7 +226,8 @@ void gemm_tr_kernel(const GemmArgs p) {
     constexpr int EPI_WNO = EPI == 1 ? WN / 2 : WN;
     constexpr int EPI_ROW_CHUNKS = EPI_WNO * 2 / 16;
     constexpr int EPI_ROWS_PER_PASS = (EPI_ROW_CHUNKS & (EPI_ROW_CHUNKS - 1)) == 0 ? 64 / EPI_ROW_CHUNKS : 4;
-    constexpr int EPI_STORES = MODE == 1 ? 0 : 2 * ((WM / 2) / EPI_ROWS_PER_PASS);
+    constexpr int EPI_PARTS = (WM / 16) % 2 == 0 ? 2 : WM / 16;       // the wave tile is staged in parts of whole m tiles
+    constexpr int EPI_STORES = MODE == 1 ? 0 : EPI_PARTS * ((WM / EPI_PARTS) / EPI_ROWS_PER_PASS);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -340,6 +341,7 @@ void gemm_tr_kernel(const GemmArgs p) {
     // With 12 chunks per k row of B one copy of the workgroup (NWAVES*64 chunks) does not end on a row
     // boundary: a lane's (k row, chunk) then differs from copy to copy and it keeps one offset per copy.
     constexpr bool B_ROWS_WHOLE = (C::NWAVES * 64) % C::CPR_B == 0;
+    constexpr bool A_ROWS_WHOLE = (C::NWAVES * 64) % C::CPR_A == 0;
     constexpr int AS_COPIES = BM / 64;
     static_assert(C::NWAVES > AS_COPIES, "some wave must be left to copy the b_scale values");
     const bool sc_is_b = wave >= AS_COPIES;                       // this wave's scale copy is the b_scale one
@@ -348,16 +350,28 @@ void gemm_tr_kernel(const GemmArgs p) {
     struct CopyPlan {
         uint32_t a_voff, b_voff, sc_voff;
         uint32_t b_voffq[C::B_LOADS];           // only without B_ROWS_WHOLE
+        uint32_t a_voffq[C::A_LOADS];           // only without A_ROWS_WHOLE
         int kb_begin;
         __amdgpu_buffer_rsrc_t b_rsrc, sc_rsrc;
     };
     auto copy_plan = [&](const Tile& t) -> CopyPlan {
         CopyPlan c;
         int P = wave * 64 + lane;
-        int krow = P / C::CPR_A, ch = (P % C::CPR_A) ^ swz_of_krow<C::CPR_A>(krow);
+        int krow = P / C::CPR_A, ch = stored_to_chunk<C::CPR_A>(P % C::CPR_A, swz_of_krow<C::CPR_A>(krow));
         int col = t.m0 + 16 * ch;
         col = col < p.lda ? col : t.m0;
         c.a_voff = (uint32_t)krow * (uint32_t)p.lda + (uint32_t)col;
+#pragma unroll
+        for (int q = 0; q < C::A_LOADS; q++) {
+            c.a_voffq[q] = 0;
+            if constexpr (!A_ROWS_WHOLE) {
+                const int Pq = q * C::NWAVES * 64 + P;
+                const int kr = Pq / C::CPR_A;
+                int cl = t.m0 + 16 * stored_to_chunk<C::CPR_A>(Pq % C::CPR_A, swz_of_krow<C::CPR_A>(kr));
+                cl = cl < p.lda ? cl : t.m0;
+                c.a_voffq[q] = (uint32_t)kr * (uint32_t)p.lda + (uint32_t)cl;
+            }
+        }
         krow = P / C::CPR_B; ch = stored_to_chunk<C::CPR_B>(P % C::CPR_B, swz_of_krow<C::CPR_B>(krow));
         col = t.n0 + 16 * ch;
         col = col < p.n ? col : t.n0;
@@ -398,7 +412,10 @@ void gemm_tr_kernel(const GemmArgs p) {
         const uint32_t sa = lds_base + stage * C::STAGE_BYTES + wave * 1024;
         const uint32_t kb = (uint32_t)(cp.kb_begin + blk);
         if constexpr (q < C::A_LOADS) {
-            copy16_global_to_lds(a_rsrc, sa + q * C::NWAVES * 1024, cp.a_voff, kb * a_kstep + (uint32_t)(q * ROWS_PER_COPY_A) * (uint32_t)p.lda);
+            if constexpr (A_ROWS_WHOLE)
+                copy16_global_to_lds(a_rsrc, sa + q * C::NWAVES * 1024, cp.a_voff, kb * a_kstep + (uint32_t)(q * ROWS_PER_COPY_A) * (uint32_t)p.lda);
+            else
+                copy16_global_to_lds(a_rsrc, sa + q * C::NWAVES * 1024, cp.a_voffq[q], kb * a_kstep);
         } else if constexpr (q < C::A_LOADS + C::B_LOADS) {
             constexpr int qb = q - C::A_LOADS;
             if constexpr (B_ROWS_WHOLE)
@@ -425,7 +442,7 @@ void gemm_tr_kernel(const GemmArgs p) {
     const int a_chunk0 = wave_m * (WM / 16), b_chunk0 = wave_n * (WN / 16);
 
     auto read_a = [&](v8i& dst, int t, const unsigned char* sbase) {
-        const unsigned char* q = sbase + a_lane_off + (((a_chunk0 + t) ^ swz_a) << 4);
+        const unsigned char* q = sbase + a_lane_off + (chunk_to_stored<C::CPR_A>(a_chunk0 + t, swz_a) << 4);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             v2i x = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_V2I(q + j * 32 * BM));
@@ -717,12 +734,12 @@ void gemm_tr_kernel(const GemmArgs p) {
         constexpr int WNO = EPI == 1 ? WN / 2 : WN;                   // output columns of the wave tile
         constexpr int ROW_CHUNKS = WNO * 2 / 16;                      // 16-byte chunks per tile row
         constexpr int ROWS_PER_SWEEP = 16 / ROW_CHUNKS > 0 ? 16 / ROW_CHUNKS : 1;
-        constexpr int HALF_ROWS = WM / 2, HALF_MT = C::MT / 2;
+        constexpr int HALF_ROWS = WM / EPI_PARTS, HALF_MT = C::MT / EPI_PARTS;    // a "half" is one of EPI_PARTS parts: two, or one per m tile if their number is odd
         // A row of 12 chunks is staged with one chunk of padding instead of the XOR swizzle: with 13
         // chunks from row to row, 16 consecutive rows of one chunk column fall on 16 different bank groups.
         constexpr bool ROW_POW2 = (ROW_CHUNKS & (ROW_CHUNKS - 1)) == 0;
         constexpr int RSTRIDE = ROW_POW2 ? WNO * 2 : WNO * 2 + 16;    // bytes from row to row in the staging area
-        static_assert(C::MT % 2 == 0 && C::NWAVES * HALF_ROWS * RSTRIDE <= C::STAGE_BYTES, "output staging must fit one stage");
+        static_assert(C::MT % EPI_PARTS == 0 && C::NWAVES * HALF_ROWS * RSTRIDE <= C::STAGE_BYTES, "output staging must fit one stage");
         unsigned char* region = lds + (NSTAGE - 1) * C::STAGE_BYTES + wave * (HALF_ROWS * RSTRIDE);
         const int ldc = EPI == 1 ? p.n / 2 : p.n;
         // Stores go through buffer descriptors: an offset of 0xFFFFFFFF drops the lane's store, so the
@@ -734,7 +751,7 @@ void gemm_tr_kernel(const GemmArgs p) {
         const int col0 = EPI == 1 ? n0 / 2 : n0;
         uint16_t* const c_tile = p.c + (size_t)m0 * ldc + col0;
 #pragma unroll
-        for (int half = 0; half < 2; half++) {
+        for (int half = 0; half < EPI_PARTS; half++) {
 #pragma unroll
             for (int th = 0; th < HALF_MT; th++) {
                 const int t = half * HALF_MT + th;
@@ -760,7 +777,7 @@ void gemm_tr_kernel(const GemmArgs p) {
             // case, a lane keeps its row-in-pass and chunk over all passes.
             constexpr int ROWS_PER_PASS = ROW_POW2 ? 64 / ROW_CHUNKS : 4, PASSES = HALF_ROWS / ROWS_PER_PASS;
             static_assert(HALF_ROWS % ROWS_PER_PASS == 0 && ROWS_PER_PASS * ROW_CHUNKS <= 64, "a half tile is a whole number of passes");
-            static_assert(MODE == 1 || EPI_STORES == 2 * PASSES, "store count used by the next tile's wait");
+            static_assert(MODE == 1 || EPI_STORES == EPI_PARTS * PASSES, "store count used by the next tile's wait");
             // lane -> (row inside the pass, chunk); everything else about a store's address is uniform
             // and sits in the descriptor, so the 16 stores need one address register, not 16
             const int lane_r = lane / ROW_CHUNKS, lane_chunk = lane % ROW_CHUNKS;

@@ -54,7 +54,8 @@ enum {
     FP8BS_VARIANT_SKINNY64x288 = 8, /* same, 288-wide tile, 3 stages                             */
     FP8BS_VARIANT_T256x192 = 9,   /* 256(m) x 192(n) tile, 8 waves: fills more CUs when n/256 rounds up badly */
     FP8BS_VARIANT_T256x128S3 = 10, /* 256 x 128 tile, three LDS stages (a copy has two K blocks' time to land) */
-    FP8BS_VARIANT_COUNT = 11
+    FP8BS_VARIANT_T192x192S3 = 11, /* 192 x 192 tile, 8 waves of 48 x 96, three LDS stages     */
+    FP8BS_VARIANT_COUNT = 12
 };
 
 /* What fp8bs_plan() decides for a shape. Replaces the exact-(m,n,k) if-ladder of the reference

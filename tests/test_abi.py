@@ -33,9 +33,9 @@ def test_plan_shape_families(pkg):
     assert p.variant == 6 and (p.tile_m, p.tile_n) == (64, 144) and p.split_k == 2 and p.grid_x == 256
     assert p.workspace_bytes == p.split_k * 64 * 18432 * 4 == pkg.workspace_bytes(64, 18432, 7168)
     p = pkg.plan(130, 190, 256)                         # n not a multiple of 8 -> a tiled kernel without a K split
-    assert p.variant in (2, 3, 4, 9, 10) and p.split_k == 1
+    assert p.variant in (2, 3, 4, 9, 10, 11) and p.split_k == 1
     p = pkg.plan(1024, 190, 7168)                       # (the same shape with n = 192 would be split)
-    assert p.variant in (2, 3, 4, 9, 10) and p.split_k == 1 and pkg.plan(1024, 192, 7168).split_k > 1
+    assert p.variant in (2, 3, 4, 9, 10, 11) and p.split_k == 1 and pkg.plan(1024, 192, 7168).split_k > 1
     for m in (130, 4095, 3, 1):                               # any m: the tiled kernels, one launch, nothing extra in the workspace
         p, q = pkg.plan(m, 192, 256), pkg.plan((m + 3) & ~3, 192, 256)
         assert p.variant == q.variant and p.variant not in (1, 6, 7, 8) and p.split_k == q.split_k
@@ -49,8 +49,10 @@ def test_plan_shape_families(pkg):
     assert p.variant in (3, 4, 10) and p.split_k > 1
     p = pkg.plan(6144, 4608, 7168)                      # large: the 256x256 tile, no split
     assert p.variant == 2 and p.split_k == 1
-    p = pkg.plan(4096, 2112, 7168)                      # 2112 = 11 x 192: 176 tiles of 256x192 instead of 144 of 256x256, 16 of them a quarter full
-    assert p.variant == 9 and (p.tile_m, p.tile_n) == (256, 192) and p.grid_x == 176 and p.lds_bytes == 2 * (128 * 448 + 1024 + 256)
+    p = pkg.plan(4096, 2112, 7168)                      # 2112 = 11 x 192: 242 tiles of 192x192 instead of 144 of 256x256, 16 of them a quarter full
+    assert p.variant == 11 and (p.tile_m, p.tile_n) == (192, 192) and p.grid_x == 242 and p.lds_bytes == 3 * (128 * 384 + 1024 + 256)
+    p = pkg.plan(4096, 3072, 8192)                      # 256 tiles of 256x192
+    assert p.variant == 9 and (p.tile_m, p.tile_n) == (256, 192) and p.grid_x == 256 and p.lds_bytes == 2 * (128 * 448 + 1024 + 256)
     p = pkg.plan(4096, 2048, 8192)                      # 256 tiles of 256x128, three stages
     assert p.variant == 10 and (p.tile_m, p.tile_n) == (256, 128) and p.lds_bytes == 3 * (128 * 384 + 1024 + 256)
 

@@ -62,14 +62,14 @@ def test_config1_and_entry_point_contract(pkg, oracle, dev):
 
 def test_golden_fixture_bit_exact(pkg, golden_gemm, dev):
     cpu, expected, _ = golden_gemm
-    for variant in (0, 1, 3, 4, 6, 7, 8, 9, 10): # planner's choice, generic, 128x128 tile, 64x128 tile, the three ring kernels, 256x192 tile, three-stage 256x128
+    for variant in (0, 1, 3, 4, 6, 7, 8, 9, 10, 11): # planner's choice, generic, 128x128 tile, 64x128 tile, the three ring kernels, 256x192 tile, three-stage 256x128
         out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1 if variant else 0)
         assert torch.equal(out.cpu().view(torch.int16), expected.view(torch.int16)), "variant %d" % variant
     out = pkg.custom_kernel(_to(cpu, dev), variant=4, split_k=2)            # exact data: split-K is exact too
     assert torch.equal(out.cpu().view(torch.int16), expected.view(torch.int16))
 
 
-@pytest.mark.parametrize("variant,split_k", [(1, 1), (2, 1), (3, 1), (4, 1), (5, 1), (6, 1), (2, 2), (3, 3), (4, 4), (5, 8), (4, 7), (6, 2), (6, 8), (7, 1), (7, 2), (7, 3), (8, 1), (8, 4), (9, 1), (9, 2), (9, 8), (10, 1), (10, 2), (10, 3), (10, 4), (10, 8)])
+@pytest.mark.parametrize("variant,split_k", [(1, 1), (2, 1), (3, 1), (4, 1), (5, 1), (6, 1), (2, 2), (3, 3), (4, 4), (5, 8), (4, 7), (6, 2), (6, 8), (7, 1), (7, 2), (7, 3), (8, 1), (8, 4), (9, 1), (9, 2), (9, 8), (10, 1), (10, 2), (10, 3), (10, 4), (10, 8), (11, 1), (11, 2), (11, 3), (11, 8)])
 def test_every_variant_and_split_on_config1(pkg, oracle, dev, variant, split_k):
     cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0])
     out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=split_k)
@@ -94,7 +94,7 @@ def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
     assert pkg.plan(m, n, k).variant != 1                       # any m and n: the vector kernels
     # every tile takes any m and n (the last bytes of a and b are repaired in LDS, a row's last chunk of
     # c is stored in pieces); the streaming kernels n % 8 == 0, and all but the planner's width m % 4 == 0
-    for variant in (2, 3, 4, 5, 9, 10) + ((6,) if n % 8 == 0 else ()) + ((7, 8) if m % 4 == 0 and n % 8 == 0 else ()):
+    for variant in (2, 3, 4, 5, 9, 10, 11) + ((6,) if n % 8 == 0 else ()) + ((7, 8) if m % 4 == 0 and n % 8 == 0 else ()):
         out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1)
         _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d" % (m, n, k, variant))
     if k >= 512 and n % 8 == 0:
@@ -107,7 +107,8 @@ def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
                                            (8192, 4096, 256, 3), (4096, 4096, 256, 4),
                                            (8192, 8256, 256, 9), (4100, 2112, 384, 9), (4096, 6336, 128, 9),
                                            (8192, 8192, 128, 10), (8192, 4096, 256, 10), (4100, 8200, 384, 10), (4096, 4096, 512, 10),
-                                           (8191, 2048, 128, 2), (4095, 2112, 384, 0), (4097, 4096, 256, 3), (4091, 4104, 128, 4), (2049, 8192, 256, 10)])
+                                           (8191, 2048, 128, 2), (4095, 2112, 384, 0), (4097, 4096, 256, 3), (4091, 4104, 128, 4), (2049, 8192, 256, 10),
+                                           (8192, 8256, 128, 11), (6144, 6144, 256, 11), (4100, 2112, 384, 11), (4095, 4232, 512, 11), (8192, 4096, 640, 11)])
 def test_many_tiles_per_workgroup_against_the_scalar_kernel(pkg, oracle, dev, m, n, k, variant):
     """Short K and a large output: every persistent workgroup walks many tiles, so the hand-over between
     tiles (next tile's first block issued ahead of the output stores, counted wait) carries the result.
@@ -215,7 +216,7 @@ def test_pointers_off_the_16_byte_grid(pkg, oracle, dev, which, shift, m, n, k):
     _check(oracle, out, ref, "misaligned %s by %d" % (which, shift))
     if "c" in which:
         assert bool((buf[:off] == -7.0).all()) and bool((buf[off + m * n:] == -7.0).all()), "bytes outside c were written"
-    for variant in (2, 4, 9, 10):
+    for variant in (2, 4, 9, 10, 11):
         out = pkg.custom_kernel((a, b, a_scale, b_scale, c), variant=variant, split_k=1)
         _check(oracle, out, ref, "misaligned %s by %d, variant %d" % (which, shift, variant))
     with pytest.raises(RuntimeError):
@@ -242,7 +243,7 @@ def test_rows_not_a_multiple_of_four_without_a_workspace(pkg, oracle, dev, m, n,
     _check(oracle, with_ws, oracle.ref_kernel(cpu), "workspace %dx%dx%d" % (m, n, k))
 
 
-@pytest.mark.parametrize("m,n,k,variant", [(130, 190, 256, 0), (64, 1001, 128, 2), (33, 257, 128, 4), (260, 2111, 256, 9), (129, 127, 384, 10), (5, 3, 128, 3)])
+@pytest.mark.parametrize("m,n,k,variant", [(130, 190, 256, 0), (64, 1001, 128, 2), (33, 257, 128, 4), (260, 2111, 256, 9), (129, 127, 384, 10), (5, 3, 128, 3), (200, 391, 512, 11)])
 def test_nothing_is_written_outside_c(pkg, oracle, dev, m, n, k, variant):
     """c sits in the middle of a larger buffer of a sentinel value: with rows that end inside a 16-byte chunk
     the kernels store the last chunk of a row in pieces, and neither the bytes in front of c nor those behind
@@ -383,7 +384,7 @@ def test_grouped_every_element_against_the_scalar_kernel(pkg, dev):
     assert int(bad.sum()) == 0, "%d elements differ, first at %s" % (int(bad.sum()), bad.nonzero()[0].tolist())
 
 
-@pytest.mark.parametrize("variant", [2, 3, 4, 5, 9, 10])
+@pytest.mark.parametrize("variant", [2, 3, 4, 5, 9, 10, 11])
 @pytest.mark.parametrize("tokens,experts,topk,n,k", [(96, 8, 2, 448, 384), (1024, 32, 8, 2112, 256), (40, 16, 1, 256, 128), (37, 8, 3, 264, 384), (341, 4, 1, 512, 128)])
 def test_grouped_with_every_tile_against_the_scalar_kernel(pkg, dev, variant, tokens, experts, topk, n, k):
     """Every tile shape in grouped mode: experts of a few rows, empty experts (40 tokens over 16 experts), expert boundaries inside a
