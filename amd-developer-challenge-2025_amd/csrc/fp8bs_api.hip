@@ -268,7 +268,7 @@ int fp8bs_gemm_grouped_ex(const void* a, const void* b, const float* a_scale, co
         variant = vector_ok ? FP8BS_VARIANT_T256x256 : FP8BS_VARIANT_GENERIC;
     } else {
         VariantInfo vi{};
-        if (!variant_info(variant, &vi) || vi.bm == 64 && vi.bn != 128) return FP8BS_ERR_BAD_VARIANT;   // no grouped mode in the streaming kernels
+        if (!variant_info(variant, &vi) || is_streaming_variant(variant)) return FP8BS_ERR_BAD_VARIANT;   // no grouped mode in the streaming kernels
         if (variant != FP8BS_VARIANT_GENERIC && !vector_ok) return FP8BS_ERR_BAD_VARIANT;
     }
     if (fp8bs::launch_gemm(variant, 2, g, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
