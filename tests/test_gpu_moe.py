@@ -43,7 +43,8 @@ def _within(oracle, out, ref, what):
     assert ok, "%s: %d elements outside the bar (max abs err %g)" % (what, nbad, maxerr)
 
 
-@pytest.mark.parametrize("m,n,k", [(256, 512, 512), (272, 288, 256), (100, 70, 128), (512, 4096, 1024)])
+@pytest.mark.parametrize("m,n,k", [(256, 512, 512), (272, 288, 256), (100, 70, 128), (512, 4096, 1024),
+                                   (257, 512, 256), (1023, 288, 384), (3, 64, 128), (130, 4096, 128)])   # rows off the 4-row grid: still the tiled kernel
 def test_dense_silu_mul(pkg, moe, oracle, mo, dev, m, n, k):
     """std 0.02 weights keep gate/up at O(1) so that silu is exercised around its bend"""
     g = torch.Generator().manual_seed(m + n)
@@ -56,9 +57,10 @@ def test_dense_silu_mul(pkg, moe, oracle, mo, dev, m, n, k):
     _within(oracle, out.cpu(), ref, "dense silu_mul %dx%dx%d" % (m, n, k))
 
 
-def test_grouped_silu_mul(pkg, moe, oracle, mo, dev):
+@pytest.mark.parametrize("tokens", [160, 161, 67])        # 480 rows; 483 and 201: totals off the 4-row grid
+def test_grouped_silu_mul(pkg, moe, oracle, mo, dev, tokens):
     cfg = pkg.inputs.CONFIGS[4]
-    data = pkg.inputs.make_grouped(cfg, tokens=160, n=512, k=256, experts=6, topk=3)
+    data = pkg.inputs.make_grouped(cfg, tokens=tokens, n=512, k=256, experts=6, topk=3)
     a, b, a_scale, b_scale, row_offsets, c = data
     rows = a.shape[0]
     h = torch.zeros(rows, 256, dtype=torch.bfloat16, device=dev)
