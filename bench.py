@@ -200,6 +200,18 @@ def main():
                                  "input_sets": nsets, "bound": "hbm", "frac": round(by / us * 1e-3 / PEAK_HBM_GBS, 4),
                                  "note": "one row: the streaming kernel with a K split of 2, then the reduction"}
         sets = None
+    # ---- configuration 2 one row and one column short: rows of a, b and c that start on odd bytes ----
+    if 2 in wanted or 3 in wanted:
+        cfg2 = pkg.inputs.CONFIGS[1]
+        ocfg = pkg.inputs.Config("odd_4095x4095x4096", cfg2.m - 1, cfg2.n - 1, cfg2.k, 0.0, 1.0, cfg2.b_std, 0, 0, cfg2.seed + 9)
+        torch.cuda.empty_cache()
+        od = gpu_dense_inputs(pkg, ocfg, dev, ocfg.seed)
+        us, us_min = time_calls(lambda i: pkg.custom_kernel(od), args.steps, args.warmup)
+        fl = 2.0 * ocfg.m * ocfg.n * ocfg.k
+        per_config[ocfg.name] = {"us": round(us, 2), "us_min": round(us_min, 2), "tflops": round(fl / us * 1e-6, 1), "bound": "mfma",
+                                 "frac": round(fl / us * 1e-6 / PEAK_FP8_TFLOPS, 4),
+                                 "note": "M % 4 != 0 and N % 8 != 0: misaligned copies, the last bytes of a and b repaired in LDS, partial chunks of c stored in pieces"}
+        od = None
     # ---- the quantisers in front of the GEMM (HBM-bound): activations of configuration 3, one expert's
     # weights of configuration 5; 4 rotating inputs (> 256 MB in total) so that reads come from HBM ----
     if args.quant:
