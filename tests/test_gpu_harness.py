@@ -63,10 +63,13 @@ def test_custom_kernel_fnuz(harness, pkg, oracle, qo, dev):
 def test_leaderboard_shape(harness, pkg, oracle, dev, case):
     """Each of the 18 shapes of the upstream benchmark (README.md:65-82), full size.  Inputs are
     N(0,1) x N(0,1): outputs are large against atol, so the FP8 matrix cores' truncated accumulation
-    shows on a few near-zero outputs; the bar is the one of configurations 1 and 2."""
+    shows on a few near-zero outputs; as for configurations 1 and 2, every element beyond the strict bar
+    must be bit-identical to the instruction-level model."""
     s = harness.LEADERBOARD_SHAPES[case]
     data = harness.generate_input(s["m"], s["n"], s["k"], s["seed"], dev)
     out = pkg.custom_kernel(data)
-    ref = oracle.ref_kernel(tuple(t.cpu() for t in data))
-    ok, nstrict, nhw = oracle.within_mfma_bar(out.cpu(), ref, RTOL, ATOL)
-    assert ok, "%s: %d strict violations, %d beyond the hardware term" % (s, nstrict, nhw)
+    cpu = tuple(t.cpu() for t in data)
+    ref = oracle.ref_kernel(cpu)
+    ok, nstrict, nunexplained = oracle.parity_report(out.cpu(), ref, cpu, pkg.plan(s["m"], s["n"], s["k"]).split_k, RTOL, ATOL)
+    print("%s: %d elements beyond the strict bar, %d not reproduced by the instruction model" % (s, nstrict, nunexplained))
+    assert ok, "%s: %d strict violations, %d not reproduced by the instruction model" % (s, nstrict, nunexplained)
