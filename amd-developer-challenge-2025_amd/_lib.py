@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(HERE, "libfp8bs.so")
 # Every symbol include/fp8bs.h declares.
 EXPORTS = (
     "fp8bs_version", "fp8bs_strerror", "fp8bs_plan", "fp8bs_workspace_bytes",
-    "fp8bs_gemm", "fp8bs_gemm_ex", "fp8bs_gemm_grouped", "fp8bs_gemm_grouped_ex",
+    "fp8bs_gemm", "fp8bs_gemm_ex", "fp8bs_gemm_noalloc", "fp8bs_gemm_grouped", "fp8bs_gemm_grouped_ex",
     "fp8bs_quantize_a", "fp8bs_quantize_b", "fp8bs_gather_a",
     "fp8bs_moe_topk", "fp8bs_moe_route_workspace_bytes", "fp8bs_moe_route",
     "fp8bs_gemm_silu_mul", "fp8bs_moe_combine", "fp8bs_convert_fnuz_to_fn",
@@ -55,6 +55,8 @@ def load() -> ctypes.CDLL:
     lib.fp8bs_workspace_bytes.argtypes = [i32, i32, i32]
     lib.fp8bs_gemm.restype = i32
     lib.fp8bs_gemm.argtypes = [vp, vp, vp, vp, vp, vp, sz, i32, i32, i32, vp]
+    lib.fp8bs_gemm_noalloc.restype = i32
+    lib.fp8bs_gemm_noalloc.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, vp]
     lib.fp8bs_gemm_ex.restype = i32
     lib.fp8bs_gemm_ex.argtypes = [vp, vp, vp, vp, vp, vp, sz, i32, i32, i32, i32, i32, vp]
     lib.fp8bs_gemm_grouped.restype = i32

@@ -164,6 +164,26 @@ bool vector_aligned(const void* a, const void* b, const void* c, const void* ws)
 
 }  // namespace
 
+// ---- built-in K-split scratch of fp8bs_gemm_noalloc ---------------------------------------------------
+// Device memory that belongs to the library's code object: every GPU the library runs on holds its own
+// copy, at its own address, until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; the address it yields (looked up once per device, with that device current) is what
+// kernels, copies and fills are given.
+static __device__ __align__(256) unsigned char scratch[FP8BS_NOALLOC_SCRATCH_BYTES];
+static void* scratch_ptr[fp8bs::MAX_DEVICES];
+
+static int scratch_address(void** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= fp8bs::MAX_DEVICES) return FP8BS_ERR_LAUNCH;
+    void* p = __atomic_load_n(&scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (!p) {
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return FP8BS_ERR_LAUNCH;
+        __atomic_store_n(&scratch_ptr[dev], p, __ATOMIC_RELEASE);     // the same value from every thread
+    }
+    *out = p;
+    return FP8BS_OK;
+}
+
 extern "C" {
 
 int fp8bs_version(void) { return 100; }
@@ -178,6 +198,7 @@ const char* fp8bs_strerror(int status) {
         case FP8BS_ERR_LAUNCH: return "kernel launch failed";
         case FP8BS_ERR_BAD_OFFSETS: return "grouped: num_experts must be positive";
         case FP8BS_ERR_BAD_VARIANT: return "unknown or inapplicable kernel variant";
+        case FP8BS_ERR_SCRATCH_LIMIT: return "fp8bs_gemm_noalloc: the K split planned for this shape needs more than the built-in scratch (FP8BS_NOALLOC_SCRATCH_BYTES); use fp8bs_gemm with a caller workspace";
         default: return "unknown fp8bs status";
     }
 }
@@ -243,6 +264,26 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
 int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
                void* c, void* ws, size_t ws_bytes, int m, int n, int k, void* stream) {
     return fp8bs_gemm_ex(a, b, a_scale, b_scale, c, ws, ws_bytes, m, n, k, FP8BS_VARIANT_AUTO, 0, stream);
+}
+
+int fp8bs_gemm_noalloc(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                       void* c, int m, int n, int k, void* stream) {
+    int st = check_common(a, b, a_scale, b_scale, c, m, n, k);
+    if (st != FP8BS_OK) return st;
+    if (m == 0 || n == 0) return FP8BS_OK;
+    // the plan fp8bs_gemm would follow; its partial planes must fit the built-in array
+    fp8bs_plan_t plan{};
+    if (k > 0) {
+        if (vector_aligned(a, b, c, nullptr)) choose(m, n, k, 0, &plan);
+        else choose_tiled(m, n, k, 0, &plan, false);
+        if (plan.split_k > 1 && plan.workspace_bytes > (uint64_t)FP8BS_NOALLOC_SCRATCH_BYTES) return FP8BS_ERR_SCRATCH_LIMIT;
+    }
+    void* ws = nullptr;
+    st = scratch_address(&ws);
+    if (st != FP8BS_OK) return st;
+    // Every partial element that the reduction reads is written by this call's main kernel first, so
+    // nothing in the array has to start at zero.
+    return fp8bs_gemm_ex(a, b, a_scale, b_scale, c, ws, (size_t)FP8BS_NOALLOC_SCRATCH_BYTES, m, n, k, FP8BS_VARIANT_AUTO, 0, stream);
 }
 
 int fp8bs_gemm_grouped_ex(const void* a, const void* b, const float* a_scale, const float* b_scale,

@@ -38,7 +38,9 @@ enum {
     FP8BS_ERR_TOO_LARGE = 4,      /* an operand exceeds the 4 GiB buffer-addressing limit    */
     FP8BS_ERR_LAUNCH = 5,         /* hipGetLastError() after launch was not hipSuccess       */
     FP8BS_ERR_BAD_OFFSETS = 6,    /* grouped: bad expert count                               */
-    FP8BS_ERR_BAD_VARIANT = 7     /* forced variant id unknown or not applicable             */
+    FP8BS_ERR_BAD_VARIANT = 7,    /* forced variant id unknown or not applicable             */
+    FP8BS_ERR_SCRATCH_LIMIT = 8   /* fp8bs_gemm_noalloc: the shape's K split needs more than
+                                     FP8BS_NOALLOC_SCRATCH_BYTES of partial planes            */
 };
 
 /* Kernel variants the planner chooses from. */
@@ -107,6 +109,20 @@ int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* 
 int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale,
                   void* c, void* ws, size_t ws_bytes, int m, int n, int k,
                   int variant, int split_k, void* stream);
+
+/* fp8bs_gemm for callers that cannot allocate device memory or hand over a workspace: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference
+ * (its split-K path allocates a tensor per call, 1-amd-fp8-mm/amd-fp8-mm-submission.py:600).  Same
+ * arguments, plan, kernels and results as fp8bs_gemm, but the fp32 partial planes of a K split live in an
+ * array of FP8BS_NOALLOC_SCRATCH_BYTES that is part of the library's device code (every GPU the library
+ * runs on holds it until the process ends).  Calls no hipMalloc / hipFree or any allocating routine.
+ * A shape whose planned K split needs more partial-plane bytes than that returns FP8BS_ERR_SCRATCH_LIMIT
+ * and launches nothing.  All calls on one GPU share the one array: calls that overlap on a GPU (two
+ * streams, two threads) race on it; calls on one stream are ordered and safe.  Nothing in the array has to
+ * be cleared between calls (every partial element read was written by the same call). */
+#define FP8BS_NOALLOC_SCRATCH_BYTES (32u * 1024u * 1024u)
+int fp8bs_gemm_noalloc(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                       void* c, int m, int n, int k, void* stream);
 
 /* Grouped (MoE expert) GEMM. Row-offset convention of 2-amd-moe/3-amd-fp8-moe-hip-myhgemm.py:142-148
  * and :328-336 (expert_offset = exclusive prefix sum of per-expert row counts), with the total
