@@ -15,7 +15,7 @@ EXPORTS = (
     "fp8bs_gemm", "fp8bs_gemm_ex", "fp8bs_gemm_noalloc", "fp8bs_gemm_grouped", "fp8bs_gemm_grouped_ex",
     "fp8bs_quantize_a", "fp8bs_quantize_b", "fp8bs_gather_a",
     "fp8bs_moe_topk", "fp8bs_moe_route_workspace_bytes", "fp8bs_moe_route",
-    "fp8bs_gemm_silu_mul", "fp8bs_moe_combine", "fp8bs_convert_fnuz_to_fn",
+    "fp8bs_gemm_silu_mul", "fp8bs_moe_combine", "fp8bs_convert_fnuz_to_fn", "fp8bs_diag_mfma_mix",
 )
 
 VARIANT_NAMES = {0: "auto", 1: "generic", 2: "t256x256", 3: "t128x128", 4: "t64x128", 5: "t256x128", 6: "skinny64x144", 7: "skinny64x256", 8: "skinny64x288", 9: "t256x192", 10: "t256x128s3", 11: "t192x192s3"}
@@ -82,6 +82,8 @@ def load() -> ctypes.CDLL:
     lib.fp8bs_moe_combine.argtypes = [vp, i32, vp, vp, vp, i32, i32, i32, vp]
     lib.fp8bs_convert_fnuz_to_fn.restype = i32
     lib.fp8bs_convert_fnuz_to_fn.argtypes = [vp, vp, sz, vp]
+    lib.fp8bs_diag_mfma_mix.restype = i32
+    lib.fp8bs_diag_mfma_mix.argtypes = [i32, i32, i32, vp, sz, vp, vp]
     _lib = lib
     return lib
 

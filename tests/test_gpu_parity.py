@@ -346,10 +346,10 @@ def test_grouped_small(pkg, oracle, dev, tokens, n, k, experts, topk):
     _check(oracle, out, oracle.ref_grouped(cpu), "grouped %s" % ((tokens, n, k, experts, topk),))
 
 
-def test_grouped_full_size_sampled_rows(pkg, oracle, dev):
-    """Configuration 5 at its published size (32 experts, 32768 routed rows, N=4096, K=7168): every
-    output row is written (no NaN left from the poison fill) and a sample of rows from every expert,
-    including first/last rows of each expert, matches the oracle on all 4096 columns."""
+def test_grouped_full_size_every_element(pkg, oracle, dev):
+    """Configuration 5 at its published size (32 experts, 32768 routed rows, N=4096, K=7168): every one of the
+    134 million outputs against the oracle (looped per expert on the host cores), and no row left unwritten
+    (no NaN left from the poison fill)."""
     cfg = pkg.inputs.CONFIGS[4]
     cpu = pkg.inputs.make_grouped(cfg)
     data = _to(cpu, dev)
@@ -358,15 +358,8 @@ def test_grouped_full_size_sampled_rows(pkg, oracle, dev):
     torch.cuda.synchronize()
     assert not bool(out.isnan().any())
     offs = cpu[4].tolist()
-    assert offs[-1] == 4096 * 8
-    g = torch.Generator().manual_seed(5)
-    rows = []
-    for e in range(32):
-        lo, hi = offs[e], offs[e + 1]
-        if hi > lo:
-            rows += [lo, hi - 1] + (torch.randint(lo, hi, (6,), generator=g)).tolist()
-    rows = torch.tensor(sorted(set(rows)))
-    _check(oracle, out[rows.to(dev)], oracle.ref_grouped(cpu, rows=rows), "config 5 sampled rows")
+    assert offs[-1] == 4096 * 8 and out.shape == (4096 * 8, 4096)
+    _check(oracle, out, oracle.ref_grouped(cpu), "config 5, all %d elements" % out.numel())
 
 
 def test_grouped_every_element_against_the_scalar_kernel(pkg, dev):
