@@ -60,10 +60,10 @@ void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out)
     out->workspace_bytes = split_k > 1 ? (uint64_t)split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
 }
 
-// Rows of c (n bf16) that keep 16-byte stores aligned: what the streaming kernels, the K split (its
-// reduction works on groups of eight outputs), the grouped walk and the fused epilogue need.  The tiled
-// kernels without a K split take any m and n (they repair the last bytes of a and b themselves and store
-// a row's last chunk of c in pieces); the streaming kernels take any m.
+// Rows of c (n bf16) that keep 16-byte stores aligned: what the streaming kernels need.  The tiled kernels
+// take any m and n in every mode (they repair the last bytes of a and b themselves, store a row's last chunk
+// of c in pieces, write the partial planes of a K split element by element where rows do not end on a
+// group of four); the streaming kernels take any m.
 bool vector_shape(int n) { return (n % 8) == 0; }
 
 // The streaming kernel is kept for what it was built for: at most 64 rows against a B too large for the
@@ -73,9 +73,8 @@ bool vector_shape(int n) { return (n % 8) == 0; }
 // second row of tiles and reads B twice.
 bool streaming_shape(int m, int n, int k) { return m <= 64 && (double)n * (double)k >= 96.0e6; }
 
-// The tile shape and K split of the tiled MFMA kernel that finish soonest (any m; any n without a split).
+// The tile shape and K split of the tiled MFMA kernel that finish soonest (any m, any n).
 void choose_tiled(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may_split = true) {
-    may_split = may_split && vector_shape(n);
     if (num_cus <= 0) num_cus = 256;
     int kbt = k / KBLK;
     // The tile shape and K split that finish soonest under a cost model in microseconds.  Per variant
@@ -135,10 +134,10 @@ void choose_streaming(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     fill_plan(m, n, k, FP8BS_VARIANT_SKINNY64x144, best_s, out);
 }
 
-// Shape-family rule.  A few rows against a very large B -> the streaming kernel.  Everything else -> the
-// tiled kernel.
-void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
-    if (vector_shape(n) && streaming_shape(m, n, k)) choose_streaming(m, n, k, num_cus, out);
+// Shape-family rule.  A few rows against a very large B -> the streaming kernel (operands on 16-byte
+// boundaries, n a multiple of 8).  Everything else -> the tiled kernel.
+void choose(int m, int n, int k, int num_cus, bool aligned, fp8bs_plan_t* out) {
+    if (aligned && vector_shape(n) && streaming_shape(m, n, k)) choose_streaming(m, n, k, num_cus, out);
     else choose_tiled(m, n, k, num_cus, out);
 }
 
@@ -156,10 +155,10 @@ int check_common(const void* a, const void* b, const float* as, const float* bs,
     return FP8BS_OK;
 }
 
-// Operands and output on 16-byte boundaries: what the streaming kernels, the K split, the grouped walk and
-// the fused epilogue need (aligned 8- and 16-byte stores of c).
-bool vector_aligned(const void* a, const void* b, const void* c, const void* ws) {
-    return ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)ws) & 15) == 0);
+// Operands and output on 16-byte boundaries: what the streaming kernels need (aligned 8- and 16-byte stores
+// of c, aligned copies).
+bool vector_aligned(const void* a, const void* b, const void* c) {
+    return ((((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15) == 0);
 }
 
 }  // namespace
@@ -206,13 +205,13 @@ const char* fp8bs_strerror(int status) {
 int fp8bs_plan(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     if (!out) return FP8BS_ERR_NULL_POINTER;
     if (m <= 0 || n <= 0 || k <= 0 || (k % KBLK) != 0) return FP8BS_ERR_BAD_SHAPE;
-    choose(m, n, k, num_cus, out);
+    choose(m, n, k, num_cus, true, out);
     return FP8BS_OK;
 }
 
 size_t fp8bs_workspace_bytes(int m, int n, int k) {
     fp8bs_plan_t p{};
-    if (fp8bs_plan(m, n, k, 0, &p) != FP8BS_OK) return 0;
+    if (fp8bs_plan(m, n, k, fp8bs::device_cus(), &p) != FP8BS_OK) return 0;
     return (size_t)p.workspace_bytes;
 }
 
@@ -225,21 +224,25 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
     hipStream_t s = (hipStream_t)stream;
     fp8bs_plan_t plan{};
     if (k == 0) variant = FP8BS_VARIANT_GENERIC;   // empty sum: the generic kernel writes zeros
-    // Operands off the 16-byte grid: the tiled kernels without a K split take them as they take rows of a, b
-    // and c that start anywhere (the same instantiation); the K split's reduction and the streaming
-    // kernels store c in aligned 8- and 16-byte pieces and are left out.  A misaligned workspace is not used.
-    const bool aligned = vector_aligned(a, b, c, nullptr);
-    if (((uintptr_t)ws & 15) != 0) { ws = nullptr; ws_bytes = 0; }
-    const bool simple = aligned && vector_shape(n);      // K split and streaming kernels possible
+    // Operands off the 16-byte grid and n off the 8-column grid: the tiled kernels take them in every mode
+    // (the same instantiation as for rows of a, b and c that start anywhere); only the streaming kernels are
+    // left out.  A workspace that starts off the 16-byte grid is used from its first 16-byte boundary on.
+    const bool aligned = vector_aligned(a, b, c);
+    if (ws && ((uintptr_t)ws & 15) != 0) {
+        const size_t skip = 16 - ((uintptr_t)ws & 15);
+        if (ws_bytes > skip) { ws = (char*)ws + skip; ws_bytes -= skip; }
+        else { ws = nullptr; ws_bytes = 0; }
+    }
+    const bool simple = aligned && vector_shape(n);      // streaming kernels possible
     if (variant == FP8BS_VARIANT_AUTO) {
-        if (aligned) choose(m, n, k, 0, &plan);
-        else choose_tiled(m, n, k, 0, &plan, false);
-        if (split_k > 1 && !simple) return FP8BS_ERR_BAD_VARIANT;
+        choose(m, n, k, fp8bs::device_cus(), aligned, &plan);
         if (split_k > 0) fill_plan(m, n, k, plan.variant, split_k, &plan);
+        // the planned K split needs a workspace the caller did not bring: the best plan that needs none
+        else if (plan.split_k > 1 && (!ws || ws_bytes < plan.workspace_bytes)) choose_tiled(m, n, k, fp8bs::device_cus(), &plan, false);
     } else {
         VariantInfo vi{};
         if (!variant_info(variant, &vi)) return FP8BS_ERR_BAD_VARIANT;
-        if (variant != FP8BS_VARIANT_GENERIC && !simple && (is_streaming_variant(variant) || split_k > 1)) return FP8BS_ERR_BAD_VARIANT;
+        if (is_streaming_variant(variant) && !simple) return FP8BS_ERR_BAD_VARIANT;
         if (is_streaming_variant(variant) && variant != FP8BS_VARIANT_SKINNY64x144 && (m % 4) != 0) return FP8BS_ERR_BAD_VARIANT;   // only the planner's width repairs a
         fill_plan(m, n, k, variant, split_k > 0 ? split_k : 1, &plan);
     }
@@ -274,8 +277,7 @@ int fp8bs_gemm_noalloc(const void* a, const void* b, const float* a_scale, const
     // the plan fp8bs_gemm would follow; its partial planes must fit the built-in array
     fp8bs_plan_t plan{};
     if (k > 0) {
-        if (vector_aligned(a, b, c, nullptr)) choose(m, n, k, 0, &plan);
-        else choose_tiled(m, n, k, 0, &plan, false);
+        choose(m, n, k, fp8bs::device_cus(), vector_aligned(a, b, c), &plan);
         if (plan.split_k > 1 && plan.workspace_bytes > (uint64_t)FP8BS_NOALLOC_SCRATCH_BYTES) return FP8BS_ERR_SCRATCH_LIMIT;
     }
     void* ws = nullptr;
@@ -300,17 +302,17 @@ int fp8bs_gemm_grouped_ex(const void* a, const void* b, const float* a_scale, co
     g.c = (uint16_t*)c; g.ws = nullptr; g.row_offsets = row_offsets;
     g.m = total_rows; g.n = n; g.k = k; g.lda = total_rows; g.nb = (n + 127) / 128;
     g.split_k = 1; g.kb_per_split = k / KBLK; g.band_h = 4; g.num_experts = num_experts;
-    const bool vector_ok = k != 0 && vector_shape(n) && vector_aligned(a, b, c, nullptr);
     if (variant == FP8BS_VARIANT_AUTO) {
         // The 256x256 tile for every routing: measured with 32 experts of 8 .. 1024 rows each (even and
         // random counts, n x k = 4096 x 7168 and 7168 x 2048) it is the fastest of the tiles throughout -
         // with few rows per expert the call streams every expert's weights once and the waves without
-        // rows only copy, and the widest tile moves the fewest bytes of a per byte of b.
-        variant = vector_ok ? FP8BS_VARIANT_T256x256 : FP8BS_VARIANT_GENERIC;
+        // rows only copy, and the widest tile moves the fewest bytes of a per byte of b.  Any n and any
+        // operand alignment (the instantiation that repairs every expert's last bytes of b).
+        variant = k != 0 ? FP8BS_VARIANT_T256x256 : FP8BS_VARIANT_GENERIC;
     } else {
         VariantInfo vi{};
         if (!variant_info(variant, &vi) || is_streaming_variant(variant)) return FP8BS_ERR_BAD_VARIANT;   // no grouped mode in the streaming kernels
-        if (variant != FP8BS_VARIANT_GENERIC && !vector_ok) return FP8BS_ERR_BAD_VARIANT;
+        if (variant != FP8BS_VARIANT_GENERIC && k == 0) return FP8BS_ERR_BAD_VARIANT;
     }
     if (fp8bs::launch_gemm(variant, 2, g, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
     return FP8BS_OK;
@@ -335,8 +337,8 @@ int fp8bs_gemm_silu_mul(const void* a, const void* b, const float* a_scale, cons
     g.m = rows; g.n = n; g.k = k; g.lda = rows; g.nb = (n + 127) / 128;
     g.split_k = 1; g.kb_per_split = k / KBLK; g.band_h = 4; g.num_experts = row_offsets ? num_experts : 0;
     g.epi = 1;
-    // 16-byte stores of n/2-wide bf16 rows need n % 16 == 0
-    int variant = (k == 0 || !vector_shape(n) || (n % 16) != 0 || !vector_aligned(a, b, h, nullptr)) ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
+    // any even n and any operand alignment: rows of h that do not keep 16-byte stores aligned are stored in pieces
+    int variant = k == 0 ? FP8BS_VARIANT_GENERIC : FP8BS_VARIANT_T256x256;
     if (fp8bs::launch_gemm(variant, row_offsets ? 2 : 0, g, (hipStream_t)stream) != hipSuccess) return FP8BS_ERR_LAUNCH;
     return FP8BS_OK;
 }

@@ -42,6 +42,17 @@ inline hipError_t raise_lds_limit(const void* kernel, int bytes, int* raised) {
     return e;
 }
 
+// CUs of the current device, asked once per device (256, MI355X's count, if the runtime does not say)
+inline int device_cus() {
+    static int cus[MAX_DEVICES];
+    const int slot = device_slot();
+    if (slot >= 0 && cus[slot] > 0) return cus[slot];
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    if (slot >= 0) cus[slot] = n;
+    return n;
+}
+
 // mode: 0 dense bf16, 1 dense split-K partials, 2 grouped.  variant: FP8BS_VARIANT_* (not AUTO).
 hipError_t launch_gemm(int variant, int mode, const GemmArgs& args, hipStream_t stream);
 // one per tile shape of the tiled kernel, each in a translation unit of its own

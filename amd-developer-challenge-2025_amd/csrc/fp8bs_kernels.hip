@@ -256,27 +256,39 @@ void gemm_skinny_kernel(const GemmArgs p) {
 // ---------------------------------------------------------------------------------------------------
 // Split-K reduction: sums `split_k` fp32 planes in a fixed order and rounds to bf16, 8 outputs per
 // thread with one 16-byte store (role of fp8_mm_128x128_ft2_split4_merge,
-// 1-amd-fp8-mm/amd-fp8-mm-submission.py:485-511, for any split count).
+// 1-amd-fp8-mm/amd-fp8-mm-submission.py:485-511, for any split count).  The planes and c are walked as flat
+// arrays of m*n elements, so the row length plays no part.  VEC: m*n is a multiple of 8 and c starts on a
+// 16-byte boundary; otherwise the same sums, element by element, with the last group cut at m*n.
 // ---------------------------------------------------------------------------------------------------
+template <bool VEC>
 __global__ __launch_bounds__(256)
 void splitk_reduce_kernel(const float* __restrict__ ws, uint16_t* __restrict__ c, size_t mn, int split_k) {
     size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 8;
     if (i >= mn) return;
-    v4f s0 = *(const v4f*)(ws + i), s1 = *(const v4f*)(ws + i + 4);
-    for (int z = 1; z < split_k; z++) {
-        s0 += *(const v4f*)(ws + (size_t)z * mn + i);
-        s1 += *(const v4f*)(ws + (size_t)z * mn + i + 4);
+    if constexpr (VEC) {
+        v4f s0 = *(const v4f*)(ws + i), s1 = *(const v4f*)(ws + i + 4);
+        for (int z = 1; z < split_k; z++) {
+            s0 += *(const v4f*)(ws + (size_t)z * mn + i);
+            s1 += *(const v4f*)(ws + (size_t)z * mn + i + 4);
+        }
+        v4i o;
+        o[0] = (int)pack_bf16x2(s0[0], s0[1]); o[1] = (int)pack_bf16x2(s0[2], s0[3]);
+        o[2] = (int)pack_bf16x2(s1[0], s1[1]); o[3] = (int)pack_bf16x2(s1[2], s1[3]);
+        *(v4i*)(c + i) = o;
+    } else {
+        const int cnt = mn - i < 8 ? (int)(mn - i) : 8;
+        for (int j = 0; j < cnt; j++) {
+            float s = ws[i + j];
+            for (int z = 1; z < split_k; z++) s += ws[(size_t)z * mn + i + j];
+            c[i + j] = (uint16_t)(pack_bf16x2(s, 0.f) & 0xFFFFu);
+        }
     }
-    v4i o;
-    o[0] = (int)pack_bf16x2(s0[0], s0[1]); o[1] = (int)pack_bf16x2(s0[2], s0[3]);
-    o[2] = (int)pack_bf16x2(s1[0], s1[1]); o[3] = (int)pack_bf16x2(s1[2], s1[3]);
-    *(v4i*)(c + i) = o;
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Generic kernel: any m, n (no alignment requirement), one output element per thread, scalar decode.
-// Only used when m or n is not a multiple of 16, where the 16-byte tile copies above cannot be used.
-// Also handles the grouped case (row_offsets != nullptr).
+// Generic kernel: any m, n (no alignment requirement), one output element per thread, scalar decode, fp32
+// accumulation.  The planner uses it for K = 0 only (an empty sum: zeros); the parity tests use it, dense and
+// grouped (row_offsets != nullptr), as the fp32-accurate HIP statement of the product.
 // ---------------------------------------------------------------------------------------------------
 __device__ __forceinline__ float e4m3fn_to_float(uint32_t v) {
     uint32_t s = (v & 0x80u) << 24, e = (v >> 3) & 15u, m = v & 7u;
@@ -378,7 +390,10 @@ hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t str
 hipError_t launch_splitk_reduce(const float* ws, uint16_t* c, size_t mn, int split_k, hipStream_t stream) {
     size_t threads = (mn + 7) / 8;
     unsigned blocks = (unsigned)((threads + 255) / 256);
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, stream, ws, c, mn, split_k);
+    if ((mn & 7) == 0 && ((uintptr_t)c & 15) == 0 && ((uintptr_t)ws & 15) == 0)
+        hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3(blocks), dim3(256), 0, stream, ws, c, mn, split_k);
+    else
+        hipLaunchKernelGGL(splitk_reduce_kernel<false>, dim3(blocks), dim3(256), 0, stream, ws, c, mn, split_k);
     return hipGetLastError();
 }
 

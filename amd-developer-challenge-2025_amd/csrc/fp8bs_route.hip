@@ -77,7 +77,8 @@ void moe_topk64_kernel(const float* __restrict__ scores, int tokens, int experts
     const int wave = blockIdx.x * (RB / 64) + (threadIdx.x >> 6), nwaves = gridDim.x * (RB / 64);
     for (int t = wave; t < tokens; t += nwaves) {
         const float v = lane < experts ? scores[(size_t)t * experts + lane] : -__builtin_inff();
-        const uint32_t u = __builtin_bit_cast(uint32_t, v);
+        uint32_t u = __builtin_bit_cast(uint32_t, v);
+        u = u == 0x80000000u ? 0u : u;              // -0.0 and +0.0 compare equal: one key, the lowest index wins
         uint32_t key = v > -__builtin_inff() ? ((u & 0x80000000u) ? ~u : (u | 0x80000000u)) : 0u;
         int mine = -1;                              // lane i keeps pick i
         for (int i = 0; i < topk; i++) {
@@ -151,6 +152,7 @@ void route_assign_kernel(const int32_t* __restrict__ top_idx, int tokens, int ex
     __shared__ int first_row[MAX_EXPERTS];       // first row of this block's tokens inside expert e's segment
     __shared__ int part[RB];
     __shared__ int tot_s[SCAN_HERE ? MAX_EXPERTS : 1], base_s[SCAN_HERE ? MAX_EXPERTS : 1];
+    int row_offsets_total;                       // row_offsets[experts]: rows that belong to some expert
     for (int i = threadIdx.x; i < experts * (RB / 32); i += RB) bits[i] = 0;
     if (SCAN_HERE) {
         // totals over all blocks and bases over the blocks before this one, summed in LDS (integer
@@ -192,8 +194,10 @@ void route_assign_kernel(const int32_t* __restrict__ top_idx, int tokens, int ex
             run += tot[i];
         }
         if (blockIdx.x == 0 && threadIdx.x == RB - 1) row_offsets[experts] = part[RB - 1];
+        row_offsets_total = part[RB - 1];
     } else {
         for (int e = threadIdx.x; e < experts; e += RB) first_row[e] = row_offsets[e] + block_base[(size_t)blockIdx.x * experts + e];
+        row_offsets_total = row_offsets[experts];
     }
     __syncthreads();
     const int t = blockIdx.x * RB + threadIdx.x;
@@ -204,6 +208,8 @@ void route_assign_kernel(const int32_t* __restrict__ top_idx, int tokens, int ex
     for (int j = 0; j < MAX_TOPK; j++)
         if (ch[j] >= 0) atomicOr(&bits[ch[j] * (RB / 32) + w], 1u << bit);
     __syncthreads();
+    // rows beyond the last expert's (they exist only if some choices were outside [0, experts)) map to no token
+    for (int r = row_offsets_total + blockIdx.x * RB + threadIdx.x; r < tokens * topk; r += gridDim.x * RB) row_map[r] = -1;
     if (t >= tokens) return;
 #pragma unroll
     for (int j = 0; j < MAX_TOPK; j++) {
@@ -291,12 +297,14 @@ extern "C" int fp8bs_moe_route(const int32_t* top_idx, int tokens, int experts, 
     if (!top_idx || !row_map) return FP8BS_ERR_NULL_POINTER;
     if (!ws || ws_bytes < fp8bs_moe_route_workspace_bytes(tokens, experts)) return FP8BS_ERR_WORKSPACE;
     hipLaunchKernelGGL(fp8bs::route_count_kernel, dim3(nblocks), dim3(fp8bs::RB), 0, s, top_idx, tokens, experts, topk, (int32_t*)ws);
+    if (hipGetLastError() != hipSuccess) return FP8BS_ERR_LAUNCH;
     if (nblocks <= 64) {
         // few blocks: every block of the assign kernel scans the counts itself
         hipLaunchKernelGGL(fp8bs::route_assign_kernel<true>, dim3(nblocks), dim3(fp8bs::RB), 0, s, top_idx, tokens, experts, topk,
                            (const int32_t*)ws, row_offsets, row_map, slot_of);
     } else {
         hipLaunchKernelGGL(fp8bs::route_scan_kernel, dim3(1), dim3(fp8bs::RB), 0, s, (int32_t*)ws, nblocks, experts, row_offsets);
+        if (hipGetLastError() != hipSuccess) return FP8BS_ERR_LAUNCH;
         hipLaunchKernelGGL(fp8bs::route_assign_kernel<false>, dim3(nblocks), dim3(fp8bs::RB), 0, s, top_idx, tokens, experts, topk,
                            (const int32_t*)ws, row_offsets, row_map, slot_of);
     }

@@ -406,6 +406,8 @@ void gemm_tr_kernel(const GemmArgs p) {
     // enforced by hand: s_waitcnt vmcnt(0) + workgroup barrier before the first read of a stage.
     const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
     constexpr int NLOADS = C::A_LOADS + C::B_LOADS + 1;     // + the scales
+    // the counted waits below name up to two blocks of copies and a tile's output stores; the counter has six bits
+    static_assert(2 * NLOADS + EPI_STORES <= 63, "vmcnt wait thresholds must fit the counter");
     // copy q (compile-time) of k block `blk` (relative to the tile's first) into `stage`
     auto issue_one = [&](const CopyPlan& cp, int stage, int blk, auto q_tag) {
         constexpr int q = decltype(q_tag)::value;
@@ -471,7 +473,7 @@ void gemm_tr_kernel(const GemmArgs p) {
     // The three candidates (byte offsets end-3 .. end-1) are worked out once, here, where registers are
     // plentiful, and kept in scalar registers.
     const bool a_tail = TAILS && (p.lda & 3) != 0 && p.k > 0;
-    const bool b_tail = TAILS && MODE != 2 && (p.n & 3) != 0 && p.k > 0;
+    const bool b_tail = TAILS && (p.n & 3) != 0 && p.k > 0;
     uint32_t acand0 = 0, acand1 = 0, acand2 = 0, a_last = 0, bcand0 = 0, bcand1 = 0, bcand2 = 0, b_last = 0;
     if (a_tail) {
         const uint32_t end = (uint32_t)p.k * (uint32_t)p.lda;
@@ -485,7 +487,7 @@ void gemm_tr_kernel(const GemmArgs p) {
         bcand0 = tail_candidate(end - 3, (uint32_t)p.n, end, (uint32_t)p.k);
         bcand1 = tail_candidate(end - 2, (uint32_t)p.n, end, (uint32_t)p.k);
         bcand2 = tail_candidate(end - 1, (uint32_t)p.n, end, (uint32_t)p.k);
-        b_last = load_last_dword(p.b + (end - 4));
+        if (MODE != 2) b_last = load_last_dword(p.b + (end - 4));     // grouped: every expert's matrix has last bytes of its own, read per tile
     }
     // (the loads are consumed here, not inside the K loop)
     acand0 = __builtin_amdgcn_readfirstlane(acand0); acand1 = __builtin_amdgcn_readfirstlane(acand1);
@@ -511,6 +513,9 @@ void gemm_tr_kernel(const GemmArgs p) {
     for (int it = 0;; it++) {
     const int m0 = cur.m0, n0 = cur.n0, kb_begin = cur.kb_begin, kb_end = cur.kb_end, split_z = cur.split_z;
     const int row_lo = cur.row_lo, row_hi = cur.row_hi;
+    if constexpr (TAILS && MODE == 2) {
+        if (b_tail) b_last = __builtin_amdgcn_readfirstlane(load_last_dword(cur.bptr + ((uint32_t)p.k * (uint32_t)p.n - 4u)));
+    }
     // a_scale: lane's output row of m-tile t is tile row wave_m*WM + 16t + i16, read from the stage's
     // copy of the a_scale row.
     // does any element of this wave's tile get stored?  (rows of the expert / matrix, columns of the matrix)
@@ -721,7 +726,15 @@ void gemm_tr_kernel(const GemmArgs p) {
             for (int u = 0; u < C::NT; u++) {
                 const int col = n0 + wave_n * WN + 16 * u + 4 * g;
                 if (col >= p.n) continue;
-                *(v4f*)(p.ws + ((size_t)split_z * p.m + row) * (size_t)p.n + col) = acc[t][u];
+                float* dst = p.ws + ((size_t)split_z * p.m + row) * (size_t)p.n + col;
+                if constexpr (!TAILS) {
+                    *(v4f*)dst = acc[t][u];
+                } else {
+                    // rows of the plane start on any 4-byte boundary and may end inside the lane's four columns
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (col + r < p.n) dst[r] = acc[t][u][r];
+                }
             }
         }
     } else {
@@ -841,17 +854,6 @@ static inline hipError_t launch_tr(const GemmArgs& a, dim3 grid, hipStream_t str
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, grid, dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
     return hipGetLastError();
-}
-
-// CUs of the current device (asked once per device)
-static inline int device_cus() {
-    static int cus[MAX_DEVICES];
-    const int slot = device_slot();
-    if (slot >= 0 && cus[slot] > 0) return cus[slot];
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    if (slot >= 0) cus[slot] = n;
-    return n;
 }
 
 template <int BM, int BN, int WM, int WN, bool WITH_EPI = false, int NSTAGE = 2>

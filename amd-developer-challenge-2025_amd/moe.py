@@ -6,45 +6,64 @@ and the host read of the counts (:230-234); here nothing synchronises with the h
 deterministic (by expert, then token id).  The outputs plug into ``quant.quantize_a(x, row_map)`` and
 ``grouped_kernel``.  No fallback: without the library the import of ``_lib`` raises.
 """
-from typing import Tuple
+from typing import Optional, Tuple
 
 import torch
 
 from . import _lib
+from .submission import _check_operands, _is_kmajor, _stream_ptr
 
 
-def topk(scores: torch.Tensor, k: int) -> torch.Tensor:
-    """scores fp32 [T, E] row-major on the GPU -> int32 [T, k], best first, lowest index first among equals."""
+_route_ws = {}     # device index -> uint8 tensor: the routing kernels' scratch, grown on demand, reused across calls
+
+
+def topk(scores: torch.Tensor, k: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """scores fp32 [T, E] row-major on the GPU -> int32 [T, k], best first, lowest index first among equals.
+    ``out`` (contiguous int32 [T, k] on the same GPU) is filled and returned if given: no allocation."""
     if scores.dtype != torch.float32 or scores.dim() != 2 or not scores.is_cuda or not scores.is_contiguous():
         raise ValueError("scores must be a contiguous float32 [tokens, experts] tensor on the GPU")
     t, e = scores.shape
-    out = torch.empty(t, k, dtype=torch.int32, device=scores.device)
+    if out is None:
+        out = torch.empty(t, k, dtype=torch.int32, device=scores.device)
+    elif out.dtype != torch.int32 or tuple(out.shape) != (t, k) or out.device != scores.device or not out.is_contiguous():
+        raise ValueError("out must be a contiguous int32 [tokens, k] tensor on the scores' device")
     with torch.cuda.device(scores.device):
-        _lib.check(_lib.load().fp8bs_moe_topk(scores.data_ptr(), t, e, k, out.data_ptr(),
-                                              torch.cuda.current_stream().cuda_stream))
+        _lib.check(_lib.load().fp8bs_moe_topk(scores.data_ptr(), t, e, k, out.data_ptr(), _stream_ptr(scores.device)))
     return out
 
 
-def route(top_idx: torch.Tensor, experts: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+def route(top_idx: torch.Tensor, experts: int, out: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None
+          ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """top_idx int32 [T, k] -> (row_offsets int32 [E+1], row_map int32 [T*k], slot_of int32 [T, k]).
 
     Expert e owns rows [row_offsets[e], row_offsets[e+1]); ``row_map[row]`` is the token of that row
     (rows of an expert ordered by token id); ``slot_of[t, j]`` is the row of token t's j-th choice.
     Rows beyond ``row_offsets[E]`` (only if some entries of ``top_idx`` are outside [0, E)) are -1.
+    ``out`` = the three tensors of a previous call (or any of those shapes, contiguous int32 on the same GPU)
+    are filled and returned: a layer that routes every step then allocates nothing per call.
     """
     if top_idx.dtype != torch.int32 or top_idx.dim() != 2 or not top_idx.is_cuda or not top_idx.is_contiguous():
         raise ValueError("top_idx must be a contiguous int32 [tokens, topk] tensor on the GPU")
     t, k = top_idx.shape
     dev = top_idx.device
-    row_offsets = torch.empty(experts + 1, dtype=torch.int32, device=dev)
-    row_map = torch.full((t * k,), -1, dtype=torch.int32, device=dev)
-    slot_of = torch.empty(t, k, dtype=torch.int32, device=dev)
+    if out is None:
+        row_offsets = torch.empty(experts + 1, dtype=torch.int32, device=dev)
+        row_map = torch.empty(t * k, dtype=torch.int32, device=dev)
+        slot_of = torch.empty(t, k, dtype=torch.int32, device=dev)
+    else:
+        row_offsets, row_map, slot_of = out
+        for name, x, shape in (("row_offsets", row_offsets, (experts + 1,)), ("row_map", row_map, (t * k,)), ("slot_of", slot_of, (t, k))):
+            if x.dtype != torch.int32 or tuple(x.shape) != shape or x.device != dev or not x.is_contiguous():
+                raise ValueError("out: %s must be a contiguous int32 tensor of shape %s on top_idx's device" % (name, shape))
+    lib = _lib.load()
+    need = lib.fp8bs_moe_route_workspace_bytes(t, experts)
+    ws = _route_ws.get(dev.index)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(max(need, 4096), dtype=torch.uint8, device=dev)
+        _route_ws[dev.index] = ws
     with torch.cuda.device(dev):
-        lib = _lib.load()
-        need = lib.fp8bs_moe_route_workspace_bytes(t, experts)
-        ws = torch.empty(max(need, 4), dtype=torch.uint8, device=dev)
         _lib.check(lib.fp8bs_moe_route(top_idx.data_ptr(), t, experts, k, row_offsets.data_ptr(), row_map.data_ptr(),
-                                       slot_of.data_ptr(), ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream))
+                                       slot_of.data_ptr(), ws.data_ptr(), ws.numel(), _stream_ptr(dev)))
     return row_offsets, row_map, slot_of
 
 
@@ -57,28 +76,35 @@ def gate_up_silu(data):
     2-amd-moe/5-amd-fp8-moe-hip-fuse.py:366-408.  Fills and returns ``h``.
     """
     a, b, a_scale, b_scale, row_offsets, h = data
+    if a.dim() != 2:
+        raise ValueError("a must be a [rows, k] tensor")
     rows, k = a.shape
     grouped = row_offsets is not None
+    if b.dim() != (3 if grouped else 2):
+        raise ValueError("b must be [E, n, k] with row_offsets and [n, k] without")
     num_experts = b.shape[0] if grouped else 0
     n = b.shape[1] if grouped else b.shape[0]
-    if a.dtype != torch.float8_e4m3fn or b.dtype != torch.float8_e4m3fn or a_scale.dtype != torch.float32 \
-            or b_scale.dtype != torch.float32 or h.dtype != torch.bfloat16:
-        raise TypeError("a, b must be float8_e4m3fn, the scales float32, h bfloat16")
-    if n % 2 or tuple(h.shape) != (rows, n // 2) or not h.is_contiguous():
-        raise ValueError("h must be a contiguous [rows, n/2] tensor")
-    if k % 128 or not a.t().is_contiguous() or not a_scale.t().is_contiguous():
-        raise ValueError("a / a_scale must be K-major with k a multiple of 128")
-    bt = b.transpose(1, 2) if grouped else b.t()
-    bst = b_scale.transpose(1, 2) if grouped else b_scale.t()
-    if not bt.is_contiguous() or not bst.is_contiguous():
-        raise ValueError("b and b_scale must be K-major (per expert)")
-    if grouped and (row_offsets.dtype != torch.int32 or tuple(row_offsets.shape) != (num_experts + 1,) or not row_offsets.is_cuda):
-        raise ValueError("row_offsets must be an int32 GPU tensor with num_experts+1 entries")
+    if n % 2:
+        raise ValueError("n must be even: gate and up rows come in pairs")
+    nb, kb = (n + 127) // 128, k // 128
+    if grouped:
+        if tuple(b.shape) != (num_experts, n, k) or tuple(b_scale.shape) != (num_experts, nb, kb):
+            raise ValueError("b / b_scale shapes do not match [E, n, k] / [E, ceil(n/128), k/128]")
+        if not b.transpose(1, 2).is_contiguous() or not b_scale.transpose(1, 2).is_contiguous():
+            raise ValueError("every expert of b and b_scale must be K-major")
+        if row_offsets.dtype != torch.int32 or tuple(row_offsets.shape) != (num_experts + 1,) or row_offsets.device != a.device:
+            raise ValueError("row_offsets must be an int32 tensor with num_experts+1 entries on the operands' GPU")
+    else:
+        if tuple(b.shape) != (n, k) or tuple(b_scale.shape) != (nb, kb):
+            raise ValueError("b / b_scale shapes do not match [n, k] / [ceil(n/128), k/128]")
+        if not _is_kmajor(b) or not _is_kmajor(b_scale):
+            raise ValueError("b and b_scale must be K-major")
+    # dtypes, devices, shapes and K-major strides of a, a_scale and h ([rows, n/2]) as for the plain GEMM's c
+    _check_operands(a, b, a_scale, b_scale, h, rows, n // 2, k)
     with torch.cuda.device(a.device):
         _lib.check(_lib.load().fp8bs_gemm_silu_mul(
             a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(), h.data_ptr(),
-            row_offsets.data_ptr() if grouped else None, num_experts, rows, n, k,
-            torch.cuda.current_stream().cuda_stream))
+            row_offsets.data_ptr() if grouped else None, num_experts, rows, n, k, _stream_ptr(a.device)))
     return h
 
 
@@ -97,5 +123,5 @@ def combine(y: torch.Tensor, slot_of: torch.Tensor, weights: torch.Tensor) -> to
     out = torch.empty(t, d, dtype=torch.bfloat16, device=y.device)
     with torch.cuda.device(y.device):
         _lib.check(_lib.load().fp8bs_moe_combine(y.data_ptr(), y.shape[0], slot_of.data_ptr(), weights.data_ptr(), out.data_ptr(),
-                                                 t, k, d, torch.cuda.current_stream().cuda_stream))
+                                                 t, k, d, _stream_ptr(y.device)))
     return out

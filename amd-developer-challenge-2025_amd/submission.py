@@ -23,14 +23,17 @@ import torch
 
 from . import _lib
 
-_workspaces = {}   # device index -> uint8 tensor, grown on demand, reused across calls
+_workspaces = {}   # (device index, stream) -> uint8 tensor, grown on demand, reused across calls on that stream
 
 
-def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    ws = _workspaces.get(device.index)
+def _workspace(device: torch.device, nbytes: int, stream: int = 0) -> torch.Tensor:
+    """The K split's partial planes: one buffer per device and stream, so that calls that overlap on two
+    streams do not write each other's planes."""
+    key = (device.index, stream)
+    ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[device.index] = ws
+        _workspaces[key] = ws
     return ws
 
 
@@ -48,12 +51,25 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 _plan_cache = {}   # (m, n, k) -> workspace bytes the planner asks for
 
 # Operands that passed the checks once: a caller that hands over the same five tensor objects again
-# (a benchmark loop, a layer called every step) skips the dtype / shape / stride checks, which cost more
-# host time than a small GEMM takes on the GPU.  An entry is keyed by the identities and version
-# counters of the tensors (any in-place change of a tensor, its metadata included, bumps the counter)
-# and holds weak references, so a recycled id() cannot alias a dead tensor.
+# (a benchmark loop, a layer called every step) skips the dtype / device / K-major checks, which cost more
+# host time than a small GEMM takes on the GPU.  An entry is keyed by the identities and version counters
+# of the tensors and holds weak references, so a recycled id() cannot alias a dead tensor; what the
+# version counter does not cover (resize_, set_, .data = ...) is caught by comparing the addresses, shapes
+# and strides kept with the entry.  Tensors without a version counter (made under inference_mode) take
+# the full checks every time.
 _CHECKED_MAX = 64
-_checked = {}      # key -> (weakrefs, m, n, k, workspace bytes, device index)
+_checked = {}      # key -> (weakrefs, (addresses, shapes, strides), m, n, k, workspace bytes, device index)
+
+
+def _cache_key(ts):
+    try:
+        return tuple(x for t in ts for x in (id(t), t._version))
+    except RuntimeError:
+        return None
+
+
+def _layout(ts):
+    return tuple(t.data_ptr() for t in ts), tuple(t.shape for t in ts), tuple(t.stride() for t in ts)
 
 
 def _stream_ptr(device: torch.device) -> int:
@@ -72,17 +88,17 @@ def _check_operands(a, b, a_scale, b_scale, c, rows, n, k):
         raise TypeError("c must be torch.bfloat16")
     if k % 128 != 0:
         raise ValueError("k must be a multiple of 128 (got %d)" % k)
-    for name, t in (("a", a), ("b", b), ("a_scale", a_scale), ("b_scale", b_scale), ("c", c)):
-        if not t.is_cuda:
-            raise ValueError("%s must be a GPU tensor: this path has no CPU implementation" % name)
-        if t.device != a.device:
-            raise ValueError("all tensors must be on the same device")
-    if a.shape[1] != k or tuple(a_scale.shape) != (rows, k // 128):
+    if a.dim() != 2 or a.shape[1] != k or tuple(a_scale.shape) != (rows, k // 128):
         raise ValueError("a / a_scale shapes do not match [rows, k] / [rows, k/128]")
     if not _is_kmajor(a) or not _is_kmajor(a_scale):
         raise ValueError("a and a_scale must be K-major (stride (1, rows)), as the reference lays them out")
     if not c.is_contiguous() or tuple(c.shape) != (rows, n):
         raise ValueError("c must be a contiguous [rows, n] tensor")
+    for name, t in (("a", a), ("b", b), ("a_scale", a_scale), ("b_scale", b_scale), ("c", c)):
+        if not t.is_cuda:
+            raise ValueError("%s must be a GPU tensor: this path has no CPU implementation" % name)
+        if t.device != a.device:
+            raise ValueError("all tensors must be on the same device")
 
 
 def plan(m: int, n: int, k: int) -> _lib.Plan:
@@ -104,20 +120,22 @@ def custom_kernel(data, variant: int = 0, split_k: int = 0):
     """
     a, b, a_scale, b_scale, c = data
     lib = _lib.load()
-    if variant == 0 and split_k == 0:
-        key = (id(a), a._version, id(b), b._version, id(a_scale), a_scale._version, id(b_scale), b_scale._version, id(c), c._version)
+    key = _cache_key(data) if variant == 0 and split_k == 0 else None
+    if key is not None:
         hit = _checked.get(key)
         if hit is not None:
-            refs, m, n, k, need, dev_index = hit
-            if refs[0]() is a and refs[1]() is b and refs[2]() is a_scale and refs[3]() is b_scale and refs[4]() is c:
+            refs, layout, m, n, k, need, dev_index = hit
+            now = _layout(data)
+            if refs[0]() is a and refs[1]() is b and refs[2]() is a_scale and refs[3]() is b_scale and refs[4]() is c \
+                    and now == layout and dev_index == torch.cuda.current_device():
+                stream = _stream_ptr(a.device)
                 ws_ptr, ws_len = None, 0
                 if need:
-                    ws = _workspace(a.device, need)
+                    ws = _workspace(a.device, need, stream)
                     ws_ptr, ws_len = ws.data_ptr(), ws.numel()
-                if dev_index == torch.cuda.current_device():
-                    _lib.check(lib.fp8bs_gemm_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(), c.data_ptr(),
-                                                 ws_ptr, ws_len, m, n, k, 0, 0, _stream_ptr(a.device)))
-                    return c
+                ptrs = now[0]
+                _lib.check(lib.fp8bs_gemm_ex(ptrs[0], ptrs[1], ptrs[2], ptrs[3], ptrs[4], ws_ptr, ws_len, m, n, k, 0, 0, stream))
+                return c
     m, k = a.shape
     n = b.shape[0]
     _check_operands(a, b, a_scale, b_scale, c, m, n, k)
@@ -131,24 +149,21 @@ def custom_kernel(data, variant: int = 0, split_k: int = 0):
         if need is None:
             need = workspace_bytes(m, n, k) if (m > 0 and n > 0 and k > 0) else 0
             _plan_cache[(m, n, k)] = need
-        if len(_checked) >= _CHECKED_MAX:
-            _checked.pop(next(iter(_checked)))
-        _checked[(id(a), a._version, id(b), b._version, id(a_scale), a_scale._version, id(b_scale), b_scale._version, id(c), c._version)] = (
-            tuple(weakref.ref(t) for t in (a, b, a_scale, b_scale, c)), m, n, k, need, a.device.index)
+        if key is not None:
+            if len(_checked) >= _CHECKED_MAX:
+                _checked.pop(next(iter(_checked)))
+            _checked[key] = (tuple(weakref.ref(t) for t in data), _layout(data), m, n, k, need, a.device.index)
     else:
         need = max(split_k, 1) * m * n * 4 if split_k > 1 else 0
-    ws_ptr, ws_len = None, 0
-    if need:
-        ws = _workspace(a.device, need)
-        ws_ptr, ws_len = ws.data_ptr(), ws.numel()
     # kernels are launched on the device the pointers live on: the library uses the current device
-    if a.device.index != torch.cuda.current_device():
-        with torch.cuda.device(a.device):
-            st = lib.fp8bs_gemm_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
-                                   c.data_ptr(), ws_ptr, ws_len, m, n, k, variant, split_k, _stream_ptr(a.device))
-    else:
+    with torch.cuda.device(a.device):
+        stream = _stream_ptr(a.device)
+        ws_ptr, ws_len = None, 0
+        if need:
+            ws = _workspace(a.device, need, stream)
+            ws_ptr, ws_len = ws.data_ptr(), ws.numel()
         st = lib.fp8bs_gemm_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
-                               c.data_ptr(), ws_ptr, ws_len, m, n, k, variant, split_k, _stream_ptr(a.device))
+                               c.data_ptr(), ws_ptr, ws_len, m, n, k, variant, split_k, stream)
     _lib.check(st)
     return c
 
@@ -164,7 +179,22 @@ def grouped_kernel(data, variant: int = 0):
     [E, ceil(n/128), k/128] with stride (nb*kb, 1, nb).  Fills and returns ``c``; no host sync.
     """
     a, b, a_scale, b_scale, row_offsets, c = data
+    lib = _lib.load()
+    key = _cache_key(data)
+    if key is not None:
+        key = ("grouped",) + key
+        hit = _checked.get(key)
+        if hit is not None:
+            refs, layout, rows, n, k, num_experts, dev_index = hit
+            now = _layout(data)
+            if all(r() is t for r, t in zip(refs, data)) and now == layout and dev_index == torch.cuda.current_device():
+                ptrs = now[0]
+                _lib.check(lib.fp8bs_gemm_grouped_ex(ptrs[0], ptrs[1], ptrs[2], ptrs[3], ptrs[5], ptrs[4], num_experts, rows, n, k,
+                                                     variant, _stream_ptr(a.device)))
+                return c
     rows, k = a.shape
+    if b.dim() != 3:
+        raise ValueError("b must be [E, n, k]")
     num_experts, n = b.shape[0], b.shape[1]
     _check_operands(a, b, a_scale, b_scale, c, rows, n, k)
     nb, kb = (n + 127) // 128, k // 128
@@ -172,12 +202,14 @@ def grouped_kernel(data, variant: int = 0):
         raise ValueError("b / b_scale shapes do not match [E, n, k] / [E, ceil(n/128), k/128]")
     if not b.transpose(1, 2).is_contiguous() or not b_scale.transpose(1, 2).is_contiguous():
         raise ValueError("every expert of b and b_scale must be K-major")
-    if row_offsets.dtype != torch.int32 or tuple(row_offsets.shape) != (num_experts + 1,) or not row_offsets.is_cuda:
-        raise ValueError("row_offsets must be an int32 GPU tensor with num_experts+1 entries")
-    lib = _lib.load()
+    if row_offsets.dtype != torch.int32 or tuple(row_offsets.shape) != (num_experts + 1,) or row_offsets.device != a.device:
+        raise ValueError("row_offsets must be an int32 tensor with num_experts+1 entries on the operands' GPU")
+    if key is not None:
+        if len(_checked) >= _CHECKED_MAX:
+            _checked.pop(next(iter(_checked)))
+        _checked[key] = (tuple(weakref.ref(t) for t in data), _layout(data), rows, n, k, num_experts, a.device.index)
     with torch.cuda.device(a.device):
-        stream = torch.cuda.current_stream().cuda_stream
         st = lib.fp8bs_gemm_grouped_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
-                                       c.data_ptr(), row_offsets.data_ptr(), num_experts, rows, n, k, variant, stream)
+                                       c.data_ptr(), row_offsets.data_ptr(), num_experts, rows, n, k, variant, _stream_ptr(a.device))
     _lib.check(st)
     return c

@@ -81,9 +81,10 @@ const char* fp8bs_strerror(int status);
 
 /* Host-only planning: no GPU needed. Replaces the dispatch of
  * 1-amd-fp8-mm/amd-fp8-mm-submission.py:528-578. `num_cus` <= 0 means 256 (MI355X).  The plan is the one
- * fp8bs_gemm follows for operands on 16-byte boundaries and a workspace of workspace_bytes; for other
- * pointers, or without that workspace when split_k > 1, fp8bs_gemm returns FP8BS_ERR_WORKSPACE in the
- * second case and runs a tiled kernel without a K split in the first. */
+ * fp8bs_gemm follows for operands on 16-byte boundaries and a workspace of workspace_bytes.  Operands off
+ * that grid get the tiled plan for the shape where this one names the streaming kernel; without the
+ * workspace of a planned K split fp8bs_gemm runs the best tiled plan that needs none (slower, same result
+ * up to the summation order). */
 int fp8bs_plan(int m, int n, int k, int num_cus, fp8bs_plan_t* out);
 
 /* Bytes of device workspace fp8bs_gemm needs for this shape (0 when split_k == 1). Replaces the
@@ -96,10 +97,11 @@ size_t fp8bs_workspace_bytes(int m, int n, int k);
  * pre-transpose branch, :570-571, overwrites a and b; this one does not).
  * Any m and n, a and b on any byte, c on any bf16 element: the tiled kernels read a and b with their
  * true row lengths, repair their last one to three bytes in LDS and, with n not a multiple of 8 or c off
- * the 16-byte grid, store c without assuming any alignment of its rows (no K split is planned then; a
- * workspace off the 16-byte grid is not used); the streaming kernel, planned for
- * at most 64 rows against a very large b with n a multiple of 8, repairs a the same way.  a_scale and
- * b_scale must be 4-byte aligned, c 2-byte aligned (FP8BS_ERR_BAD_SHAPE otherwise). */
+ * the 16-byte grid, store c (and the partial planes of a K split) without assuming any alignment of its
+ * rows; a workspace off the 16-byte grid is used from its first 16-byte boundary on; the streaming
+ * kernel, planned for at most 64 rows against a very large b with n a multiple of 8 and operands on
+ * 16-byte boundaries, repairs a the same way.  a_scale and b_scale must be 4-byte aligned, c 2-byte
+ * aligned (FP8BS_ERR_BAD_SHAPE otherwise). */
 int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
                void* c, void* ws, size_t ws_bytes, int m, int n, int k, void* stream);
 
@@ -138,7 +140,7 @@ int fp8bs_gemm_grouped(const void* a, const void* b, const float* a_scale, const
 
 /* Same with the tile forced: one of the FP8BS_VARIANT_T* tiles or FP8BS_VARIANT_GENERIC (the streaming
  * variants have no grouped mode: FP8BS_ERR_BAD_VARIANT).  FP8BS_VARIANT_AUTO reproduces
- * fp8bs_gemm_grouped (the 256x256 tile, or the scalar kernel for shapes and pointers off the 16-byte grid). */
+ * fp8bs_gemm_grouped (the 256x256 tile for any n and any operand alignment; the scalar kernel only for k = 0). */
 int fp8bs_gemm_grouped_ex(const void* a, const void* b, const float* a_scale, const float* b_scale,
                           void* c, const int32_t* row_offsets, int num_experts, int total_rows,
                           int n, int k, int variant, void* stream);
@@ -200,7 +202,7 @@ size_t fp8bs_moe_route_workspace_bytes(int tokens, int experts);
  *   row_map     [tokens*topk] row_map[row] = token that fills that row; rows of an expert are ordered by
  *                              token id (the reference hands positions out by atomicAdd, :107-156, so its
  *                              order varies between runs) - what fp8bs_quantize_a takes as its gather list;
- *                              entries beyond row_offsets[experts] are not written
+ *                              entries beyond row_offsets[experts] are set to -1
  *   slot_of     [tokens][topk] row of every (token, choice), -1 for ignored entries; may be NULL
  * experts <= 1024, topk <= 16. */
 int fp8bs_moe_route(const int32_t* top_idx, int tokens, int experts, int topk, int32_t* row_offsets,
@@ -226,10 +228,10 @@ int fp8bs_moe_combine(const void* y, int rows, const int32_t* slot_of, const flo
 /* ---- Measurement aid -------------------------------------------------------------------------------
  * No counterpart in the reference and no part of any GEMM call: runs, `iters` times per wave, the
  * instruction mix of one K block of the 256x256 tile's wave (32 FP8 MFMAs on random operands, 8 waves per
- * workgroup) with the parts selected by the bits of `mix`: 1 = the scale fold (4 v_fma per MFMA), 2 = the
- * transposing LDS reads (48 per 32 MFMAs), 4 = the global->LDS copies (8 KiB per wave per 32 MFMAs; the 8
- * workgroups an XCD runs side by side share a stream, the streams walk src cyclically) - without barriers,
- * waits or output.  One iteration is 2048 clocks of matrix-core work per SIMD, so
+ * workgroup) with the parts selected by the bits of `mix` (0 .. 15): 1 = the scale fold (4 v_fma per MFMA),
+ * 2 = the transposing LDS reads (48 per 32 MFMAs), 4 = the global->LDS copies (8 KiB per wave per 32 MFMAs;
+ * the 8 workgroups an XCD runs side by side share a stream, the streams walk src cyclically), 8 = the same
+ * multiply-accumulates as 16 MFMAs of the 32x32x64 form - without barriers, waits or output.  One iteration is 2048 clocks of matrix-core work per SIMD, so
  * iters * 2048 / 2.4e9 / time is the fraction of the nominal FP8 peak the mix reaches on `workgroups` CUs.
  * src: device buffer of src_bytes (a power of two >= 4 MiB, 16-byte aligned) whose first 64 KiB hold e4m3fn
  * codes used as operands; sink: 4 writable device bytes (never written in practice).  bench.py

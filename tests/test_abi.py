@@ -1,6 +1,7 @@
 """The C-ABI library loads without a GPU, exports every symbol include/fp8bs.h declares, and its
 host-only entry points (planner, argument checks, error strings) behave.  No GPU compute here."""
 import ctypes
+import importlib
 import os
 import re
 
@@ -32,10 +33,11 @@ def test_plan_shape_families(pkg):
     p = pkg.plan(64, 18432, 7168)                       # skinny-M: streaming tile, split-K fills the CUs
     assert p.variant == 6 and (p.tile_m, p.tile_n) == (64, 144) and p.split_k == 2 and p.grid_x == 256
     assert p.workspace_bytes == p.split_k * 64 * 18432 * 4 == pkg.workspace_bytes(64, 18432, 7168)
-    p = pkg.plan(130, 190, 256)                         # n not a multiple of 8 -> a tiled kernel without a K split
+    p = pkg.plan(130, 190, 256)                         # n not a multiple of 8, short K -> a tiled kernel without a K split
     assert p.variant in (2, 3, 4, 9, 10, 11) and p.split_k == 1
-    p = pkg.plan(1024, 190, 7168)                       # (the same shape with n = 192 would be split)
-    assert p.variant in (2, 3, 4, 9, 10, 11) and p.split_k == 1 and pkg.plan(1024, 192, 7168).split_k > 1
+    p, q = pkg.plan(1024, 190, 7168), pkg.plan(1024, 192, 7168)   # long K, few tiles: a K split, also with n off the 8-column grid
+    assert p.variant == q.variant and p.variant in (2, 3, 4, 9, 10, 11) and p.split_k == q.split_k > 1
+    assert p.workspace_bytes == p.split_k * 1024 * 190 * 4
     for m in (130, 4095, 3, 1):                               # any m: the tiled kernels, one launch, nothing extra in the workspace
         p, q = pkg.plan(m, 192, 256), pkg.plan((m + 3) & ~3, 192, 256)
         assert p.variant == q.variant and p.variant not in (1, 6, 7, 8) and p.split_k == q.split_k
@@ -90,8 +92,8 @@ def test_argument_errors_are_reported_before_any_launch(pkg):
     assert lib.fp8bs_gemm(one, one, one, one, one, None, 0, 0, 16, 128, None) == 0       # empty: nothing to do
     assert lib.fp8bs_gemm(one, one, one, one, one, None, 0, 1 << 20, 16, 1 << 13, None) == 4   # 2^33 bytes of a
     assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 16, 16, 128, 99, 1, None) == 7
-    assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 128, 20, 128, 2, 2, None) == 7  # a K split needs n % 8 == 0
-    assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 128, 20, 128, 6, 1, None) == 7  # and so do the streaming kernels
+    assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 128, 20, 512, 2, 2, None) == 3  # a K split takes any n, but needs its workspace
+    assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 128, 20, 128, 6, 1, None) == 7  # the streaming kernels need n % 8 == 0
     assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 130, 16, 128, 7, 1, None) == 7  # the wider streaming kernels need m % 4 == 0
     assert lib.fp8bs_gemm_ex(one, one, one, one, one, None, 0, 64, 256, 1024, 4, 4, None) == 3 # split-K without workspace
     assert lib.fp8bs_gemm_grouped(one, one, one, one, one, None, 4, 16, 16, 128, None) == 1
@@ -110,6 +112,40 @@ def test_custom_kernel_validates_its_operands(pkg):
         pkg.custom_kernel((a.float(), b, a_scale, b_scale, c))
     with pytest.raises(TypeError):
         pkg.custom_kernel((a, b, a_scale, b_scale, c.float()))
+
+
+def test_gate_up_silu_validates_its_operands(pkg):
+    """Wrong shapes and layouts are refused on the host: the kernel sizes its buffer descriptors from the
+    arguments, so a mismatched b or b_scale would be read past its allocation."""
+    moe = importlib.import_module("amd-developer-challenge-2025_amd.moe")
+    a, b, a_scale, b_scale, c = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0], m=32, n=128, k=256)
+    h = torch.empty(32, 64, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="GPU tensor"):
+        moe.gate_up_silu((a, b, a_scale, b_scale, None, h))                       # everything right but the device
+    wrong_k = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0], m=32, n=128, k=128)
+    with pytest.raises(ValueError, match="shapes do not match"):
+        moe.gate_up_silu((a, wrong_k[1], a_scale, b_scale, None, h))              # b's K differs from a's
+    with pytest.raises(ValueError, match="shapes do not match"):
+        moe.gate_up_silu((a, b, a_scale, wrong_k[3], None, h))                    # b_scale of another K
+    with pytest.raises(ValueError, match="shapes do not match"):
+        moe.gate_up_silu((a, b, wrong_k[2], b_scale, None, h))                    # a_scale of another K
+    with pytest.raises(ValueError, match="K-major"):
+        moe.gate_up_silu((a, b.contiguous(), a_scale, b_scale, None, h))          # row-major b
+    with pytest.raises(ValueError, match=r"\[rows, n\]"):
+        moe.gate_up_silu((a, b, a_scale, b_scale, None, torch.empty(32, 128, dtype=torch.bfloat16)))   # h must have n/2 columns
+    with pytest.raises(ValueError, match="E, n, k"):
+        moe.gate_up_silu((a, b, a_scale, b_scale, torch.zeros(2, dtype=torch.int32), h))   # grouped call with a 2-D b
+    with pytest.raises(TypeError):
+        moe.gate_up_silu((a.float(), b, a_scale, b_scale, None, h))
+
+
+def test_custom_kernel_without_version_counters(pkg):
+    """Tensors made under inference_mode have no version counter: the checked-once cache must step aside,
+    not raise (the call then fails on the operands being CPU tensors, like any other CPU call)."""
+    with torch.inference_mode():
+        data = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0], m=32, n=128, k=128)
+        with pytest.raises(ValueError, match="GPU tensor"):
+            pkg.custom_kernel(data)
 
 
 def test_root_submission_module_reexports_entry_point(pkg):

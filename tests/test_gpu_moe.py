@@ -44,7 +44,8 @@ def _within(oracle, out, ref, what):
 
 
 @pytest.mark.parametrize("m,n,k", [(256, 512, 512), (272, 288, 256), (100, 70, 128), (512, 4096, 1024),
-                                   (257, 512, 256), (1023, 288, 384), (3, 64, 128), (130, 4096, 128)])   # rows off the 4-row grid: still the tiled kernel
+                                   (257, 512, 256), (1023, 288, 384), (3, 64, 128), (130, 4096, 128),      # rows off the 4-row grid
+                                   (300, 380, 256), (129, 2002, 128), (64, 6, 128), (513, 1038, 384)])     # n/2 off the 8-column grid: rows of h stored in pieces
 def test_dense_silu_mul(pkg, moe, oracle, mo, dev, m, n, k):
     """std 0.02 weights keep gate/up at O(1) so that silu is exercised around its bend"""
     g = torch.Generator().manual_seed(m + n)
@@ -57,16 +58,17 @@ def test_dense_silu_mul(pkg, moe, oracle, mo, dev, m, n, k):
     _within(oracle, out.cpu(), ref, "dense silu_mul %dx%dx%d" % (m, n, k))
 
 
-@pytest.mark.parametrize("tokens", [160, 161, 67])        # 480 rows; 483 and 201: totals off the 4-row grid
-def test_grouped_silu_mul(pkg, moe, oracle, mo, dev, tokens):
+@pytest.mark.parametrize("tokens,n", [(160, 512), (161, 512), (67, 512),        # 480 rows; 483 and 201: totals off the 4-row grid
+                                      (160, 380), (67, 2002), (161, 262)])      # n/2 off the 8-column grid, n off the 4-byte grid of b's rows
+def test_grouped_silu_mul(pkg, moe, oracle, mo, dev, tokens, n):
     cfg = pkg.inputs.CONFIGS[4]
-    data = pkg.inputs.make_grouped(cfg, tokens=tokens, n=512, k=256, experts=6, topk=3)
+    data = pkg.inputs.make_grouped(cfg, tokens=tokens, n=n, k=256, experts=6, topk=3)
     a, b, a_scale, b_scale, row_offsets, c = data
     rows = a.shape[0]
-    h = torch.zeros(rows, 256, dtype=torch.bfloat16, device=dev)
+    h = torch.zeros(rows, n // 2, dtype=torch.bfloat16, device=dev)
     out = moe.gate_up_silu((a.to(dev), b.to(dev), a_scale.to(dev), b_scale.to(dev), row_offsets.to(dev), h))
     offs = row_offsets.tolist()
-    ref = torch.empty(rows, 256, dtype=torch.bfloat16)
+    ref = torch.empty(rows, n // 2, dtype=torch.bfloat16)
     for e in range(6):
         if offs[e + 1] > offs[e]:
             sl = slice(offs[e], offs[e + 1])

@@ -99,9 +99,11 @@ def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
     for variant in (2, 3, 4, 5, 9, 10, 11) + ((6,) if n % 8 == 0 else ()) + ((7, 8) if m % 4 == 0 and n % 8 == 0 else ()):
         out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1)
         _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d" % (m, n, k, variant))
-    if k >= 512 and n % 8 == 0:
-        for variant in (4, 6):
-            out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=2)  # the repair happens in the last split only
+    if k >= 256:
+        # a K split on any n (partial planes written element by element where rows end inside a group of four,
+        # reduction over the flat m*n array); the repair of a and b happens in the last split only
+        for variant in (4, 2, 11) + ((6,) if n % 8 == 0 else ()):
+            out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=2)
             _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d split 2" % (m, n, k, variant))
 
 
@@ -200,8 +202,8 @@ def _shifted(t, nbytes):
 @pytest.mark.parametrize("which,shift", [("a", 4), ("a", 1), ("b", 8), ("b", 3), ("c", 2), ("c", 6), ("abc", 5)])
 @pytest.mark.parametrize("m,n,k", [(64, 128, 256), (300, 520, 384), (129, 263, 128)])
 def test_pointers_off_the_16_byte_grid(pkg, oracle, dev, which, shift, m, n, k):
-    """Operands that start anywhere (a, b on any byte, c on any bf16 element): the tiled kernels take them
-    without a K split; the streaming kernels and a forced K split are refused; nothing outside c is written."""
+    """Operands that start anywhere (a, b on any byte, c on any bf16 element): the tiled kernels take them,
+    with and without a K split; the streaming kernels are refused; nothing outside c is written."""
     cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[2], m=m, n=n, k=k)
     a, b, a_scale, b_scale, c = _to(cpu, dev)
     if "a" in which:
@@ -223,8 +225,13 @@ def test_pointers_off_the_16_byte_grid(pkg, oracle, dev, which, shift, m, n, k):
         _check(oracle, out, ref, "misaligned %s by %d, variant %d" % (which, shift, variant))
     with pytest.raises(RuntimeError):
         pkg.custom_kernel((a, b, a_scale, b_scale, c), variant=6, split_k=1)     # the streaming kernels store c in aligned pieces
-    with pytest.raises(RuntimeError):
-        pkg.custom_kernel((a, b, a_scale, b_scale, c), variant=4, split_k=2)     # and so does the reduction of a K split
+    if k >= 256:
+        for variant, split in ((4, 2), (2, 3)):
+            c.fill_(float("nan"))
+            out = pkg.custom_kernel((a, b, a_scale, b_scale, c), variant=variant, split_k=split)
+            _check(oracle, out, ref, "misaligned %s by %d, variant %d, K split %d" % (which, shift, variant, split))
+        if "c" in which:
+            assert bool((buf[:off] == -7.0).all()) and bool((buf[off + m * n:] == -7.0).all()), "bytes outside c were written by the reduction"
 
 
 @pytest.mark.parametrize("m,n,k", [(5, 264, 384), (3, 264, 384), (131, 1024, 256), (1027, 136, 256)])
@@ -364,19 +371,53 @@ def test_grouped_full_size_every_element(pkg, oracle, dev):
 
 def test_grouped_every_element_against_the_scalar_kernel(pkg, dev):
     """Configuration 5's routing and shapes with K = 256: ~2300 tiles over 256 persistent workgroups.  The
-    whole output is compared with the scalar kernel's (taken by handing over a c that starts off the
-    16-byte grid)."""
+    whole output is compared with the scalar kernel's; so is the output into a c that starts off the
+    16-byte grid (the instantiation that stores rows of c in pieces), which must match the aligned call bit
+    for bit."""
     cfg = pkg.inputs.CONFIGS[4]
     data = list(_to(pkg.inputs.make_grouped(cfg, k=256), dev))
     data[5].fill_(float("nan"))
     out = pkg.grouped_kernel(tuple(data)).float()
-    scalar = list(data)
-    scalar[5] = _shifted(torch.full_like(data[5], float("nan")), 2)
-    assert scalar[5].data_ptr() % 16 != 0
-    ref = pkg.grouped_kernel(tuple(scalar)).float()
+    ref = pkg.grouped_kernel(tuple(data[:5]) + (torch.full_like(data[5], float("nan")),), variant=1).float()
     assert not bool(ref.isnan().any()) and not bool(out.isnan().any())
     bad = ~((out - ref).abs() <= ATOL + RTOL * ref.abs())
     assert int(bad.sum()) == 0, "%d elements differ, first at %s" % (int(bad.sum()), bad.nonzero()[0].tolist())
+    shifted = list(data)
+    shifted[5] = _shifted(torch.full_like(data[5], float("nan")), 2)
+    assert shifted[5].data_ptr() % 16 != 0
+    out2 = pkg.grouped_kernel(tuple(shifted)).float()
+    assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("variant", [0, 2, 3, 4, 5, 9, 10, 11])
+@pytest.mark.parametrize("tokens,experts,topk,n,k,shift", [(96, 8, 2, 190, 384, 0), (300, 5, 3, 1001, 256, 0), (37, 8, 3, 257, 128, 0),
+                                                           (341, 4, 1, 2047, 128, 0), (130, 6, 2, 262, 256, 0), (96, 8, 2, 448, 384, 3), (200, 3, 2, 263, 256, 5)])
+def test_grouped_with_columns_off_the_8_column_grid_and_pointers_off_the_16_byte_grid(pkg, oracle, dev, variant, tokens, experts, topk, n, k, shift):
+    """The grouped walk on the vector kernels with any n and any operand alignment: every expert's matrix of b
+    loses its own last bytes when n is not a multiple of four (repaired per tile), rows of c are stored in
+    pieces.  Every element against the oracle, and the library's choice must be the 256x256 tile's result bit
+    for bit (not the scalar kernel's).  A poisoned margin around c stays untouched."""
+    cfg = pkg.inputs.CONFIGS[4]
+    cpu = pkg.inputs.make_grouped(cfg, tokens=tokens, experts=experts, topk=topk, n=n, k=k)
+    a, b, a_scale, b_scale, row_offsets, c = _to(cpu, dev)
+    rows = a.shape[0]
+    if shift:
+        a = _shifted(a, shift)
+        flat = torch.empty(b.numel() + 256, dtype=torch.uint8, device=dev)
+        bv = flat[shift:shift + b.numel()].view(torch.float8_e4m3fn).view(experts, k, n)
+        bv.copy_(b.transpose(1, 2))
+        b = bv.transpose(1, 2)
+    buf = torch.full((rows * n + 256,), -7.0, dtype=torch.bfloat16, device=dev)
+    off = 64 + shift
+    c = buf[off:off + rows * n].view(rows, n)
+    ref = oracle.ref_grouped(cpu)
+    out = pkg.grouped_kernel((a, b, a_scale, b_scale, row_offsets, c), variant=variant)
+    torch.cuda.synchronize()
+    _check(oracle, out, ref, "grouped n=%d shift=%d variant %d" % (n, shift, variant))
+    assert bool((buf[:off] == -7.0).all()) and bool((buf[off + rows * n:] == -7.0).all()), "bytes outside c were written"
+    if variant == 0:
+        big = pkg.grouped_kernel((a, b, a_scale, b_scale, row_offsets, torch.empty_like(out)), variant=2)
+        assert torch.equal(out.view(torch.int16), big.view(torch.int16)), "the library's choice is not the 256x256 tile"
 
 
 @pytest.mark.parametrize("variant", [2, 3, 4, 5, 9, 10, 11])

@@ -52,6 +52,48 @@ def test_topk_rows_of_minus_inf(moe, ro, dev):
     assert got[0].tolist() == [-1, -1, -1] and got[1].tolist() == [4, -1, -1]
 
 
+@pytest.mark.parametrize("experts", [8, 32, 64, 100])          # the wave-per-token kernel (<= 64 experts) and the per-thread scan
+def test_topk_signed_zeros_compare_equal(moe, ro, dev, experts):
+    """+0.0 and -0.0 are equal scores (the reference compares with __hgt, 2-amd-moe/amd-moe-submission.py:32-56):
+    among them the lowest index wins, whatever their sign bits, in both kernels."""
+    s = torch.full((6, experts), -1.0)
+    s[0, 5], s[0, 2] = -0.0, 0.0                                 # +0 at the lower index
+    s[1, 2], s[1, 5] = -0.0, 0.0                                 # -0 at the lower index: still index 2 first
+    s[2, 1], s[2, 3], s[2, 6] = 0.0, -0.0, 0.0
+    s[3, :] = -0.0
+    s[4, :] = 0.0
+    s[4, 1::2] = -0.0
+    s[5, 7], s[5, 0], s[5, 4] = 1.0, -0.0, 0.0
+    got = moe.topk(s.to(dev), 4).cpu().numpy()
+    assert np.array_equal(got, ro.topk_ref(s.numpy(), 4))
+    assert got[0, :2].tolist() == [2, 5] and got[1, :2].tolist() == [2, 5] and got[2, :3].tolist() == [1, 3, 6]
+    assert got[3].tolist() == [0, 1, 2, 3] and got[4].tolist() == [0, 1, 2, 3] and got[5, :3].tolist() == [7, 0, 4]
+
+
+def test_route_into_caller_tensors_and_rows_beyond_the_total(moe, ro, dev):
+    """`out=`: the three outputs of an earlier call are filled again, no allocation; rows beyond
+    row_offsets[E] (choices outside [0, E)) read -1 although the tensors held other values before."""
+    rng = np.random.default_rng(5)
+    tokens, experts, k = 700, 16, 4
+    top = np.stack([rng.permutation(experts)[:k] for _ in range(tokens)]).astype(np.int32)
+    first = moe.route(torch.from_numpy(top).to(dev), experts)
+    ptrs = [t.data_ptr() for t in first]
+    top2 = top.copy()
+    top2[::3, 1] = experts + 5                                   # ignored choices: fewer rows than tokens * k
+    top2[::5, 2] = -1
+    for t in first:
+        t.fill_(12345)
+    again = moe.route(torch.from_numpy(top2).to(dev), experts, out=first)
+    assert [t.data_ptr() for t in again] == ptrs
+    wo, wm, ws = ro.route_ref(top2, experts)
+    assert np.array_equal(again[0].cpu().numpy(), wo) and np.array_equal(again[1].cpu().numpy(), wm) and np.array_equal(again[2].cpu().numpy(), ws)
+    assert int(wo[-1]) < tokens * k and bool((again[1][int(wo[-1]):] == -1).all())
+    idx = moe.topk(torch.rand(tokens, experts, device=dev), k)
+    assert moe.topk(torch.rand(tokens, experts, device=dev), k, out=idx).data_ptr() == idx.data_ptr()
+    with pytest.raises(ValueError):
+        moe.route(torch.from_numpy(top).to(dev), experts, out=(first[0], first[1][:-1], first[2]))
+
+
 @pytest.mark.parametrize("tokens,experts,k", [(300, 8, 3), (4096, 32, 8), (255, 1, 1), (1025, 1000, 4), (5, 32, 8), (20000, 16, 2)])
 def test_route_bit_exact(moe, ro, dev, tokens, experts, k):
     rng = np.random.default_rng(tokens * 31 + experts)

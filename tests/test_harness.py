@@ -31,3 +31,13 @@ def test_leaderboard_shapes(harness, pkg):
     # every one of them is planned onto a tiled MFMA kernel, none onto the scalar fallback
     for s in shapes:
         assert pkg.plan(s["m"], s["n"], s["k"]).variant != 1
+
+
+def test_main_usage_errors_need_no_gpu(harness, tmp_path, capsys):
+    """The command line of the two upstream modes: bad usage is reported before anything touches the GPU."""
+    f = tmp_path / "tests"
+    f.write_text("m: 64; n: 128; k: 256; seed: 1\n")
+    assert harness.main([]) == 2
+    assert harness.main(["rank", str(f)]) == 2
+    assert harness.main(["test", str(f)]) == 2                    # test mode without a checker: nothing to compare with
+    assert "checker" in capsys.readouterr().err

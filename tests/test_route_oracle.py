@@ -31,6 +31,10 @@ def test_topk_tie_fixture_and_special_values(ro):
     assert got[2].tolist() == [1, 4, -1, -1]                  # -inf and NaN are never selected
     sel = np.take_along_axis(s[:2], got[:2], axis=1)
     assert np.all(np.diff(sel, axis=1) <= 0)                  # best first
+    # +0.0 and -0.0 are equal scores: the lowest index wins whatever the sign bits
+    z = np.array([[-1, -1, 0.0, -1, -1, -0.0], [-1, -1, -0.0, -1, -1, 0.0], [-0.0, 0.0, -0.0, 0.0, 1.0, -1]], dtype=np.float32)
+    assert ro.topk_ref(z, 2)[0].tolist() == [2, 5] and ro.topk_ref(z, 2)[1].tolist() == [2, 5]
+    assert ro.topk_ref(z, 4)[2].tolist() == [4, 0, 1, 2]
 
 
 def test_route_matches_the_independent_torch_derivation(ro, pkg):
