@@ -47,20 +47,27 @@ def algorithmic_bytes(m, n, k):
 PREHEAT_S = 0.05              # untimed calls for at least this long before anything is timed
 
 
-def preheat(fn, seconds=PREHEAT_S):
-    """Back-to-back calls for at least `seconds` of GPU time (untimed); returns how many were made."""
+def preheat(fn, seconds=PREHEAT_S, max_seconds=1.0):
+    """Back-to-back calls (untimed) until the clocks have settled: at least `seconds` of GPU time, and on until
+    two successive chunks of ~10 ms agree within 2 % per call (out of the idle state the board first runs slow
+    for some tens of milliseconds), at most `max_seconds`.  Returns how many calls were made."""
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    done, n = 0, 8
-    e0.record()
+    done, n, total, prev = 0, 16, 0.0, None
     while True:
+        e0.record()
         for _ in range(n):
             fn(done)
             done += 1
         e1.record()
         e1.synchronize()
-        if e0.elapsed_time(e1) * 1e-3 >= seconds or done > 200000:
+        chunk = e0.elapsed_time(e1) * 1e-3
+        total += chunk
+        per_call = chunk / n
+        settled = prev is not None and abs(per_call - prev) <= 0.02 * prev
+        if (total >= seconds and settled) or total >= max_seconds or done > 500000:
             return done
-        n *= 2
+        prev = per_call if chunk >= 0.004 else None          # a chunk shorter than 4 ms is no yardstick
+        n = max(16, min(int(0.01 / max(per_call, 1e-7)), 100000))
 
 
 def time_calls(fn, steps, warmup, batches=5):

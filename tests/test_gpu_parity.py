@@ -270,6 +270,25 @@ def test_nothing_is_written_outside_c(pkg, oracle, dev, m, n, k, variant):
     _check(oracle, out, oracle.ref_kernel(cpu), "sentinel %dx%dx%d variant %d" % (m, n, k, variant))
 
 
+def test_streaming_kernel_every_row_count_up_to_48(pkg, oracle, dev):
+    """The streaming kernel multiplies only the 16-row m tiles that exist (a compile-time count per launch:
+    1, 2 or 3 for at most 48 rows).  Every row count from 1 to 48, with and without a K split, against the
+    oracle and against the scalar HIP kernel on every element."""
+    cfg = pkg.inputs.CONFIGS[2]
+    n, k = 288, 512                                               # two 144-column tiles, four K blocks
+    for m in range(1, 49):
+        cpu = pkg.inputs.make_dense(cfg, m=m, n=n, k=k)
+        data = _to(cpu, dev)
+        ref = oracle.ref_kernel(cpu)
+        scalar = pkg.custom_kernel(tuple(data[:4]) + (torch.empty_like(data[4]),), variant=1, split_k=1).float()
+        for split in (1, 2):
+            c = torch.full_like(data[4], float("nan"))
+            out = pkg.custom_kernel(tuple(data[:4]) + (c,), variant=6, split_k=split)
+            _check(oracle, out, ref, "streaming kernel, %d rows, K split %d" % (m, split))
+            bad = ~((out.float() - scalar).abs() <= ATOL + RTOL * scalar.abs())
+            assert int(bad.sum()) == 0, "%d rows, split %d: %d elements differ from the scalar kernel" % (m, split, int(bad.sum()))
+
+
 @pytest.mark.parametrize("m", [1, 3, 5, 18, 63])
 def test_decode_rows_against_a_large_b(pkg, oracle, dev, m):
     """A few token rows against configuration 4's weights (132 MB): the streaming kernel with a K split,
