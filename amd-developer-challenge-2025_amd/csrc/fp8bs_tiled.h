@@ -847,7 +847,9 @@ static inline hipError_t launch_tr(const GemmArgs& a, dim3 grid, hipStream_t str
     // rows of a that are not a multiple of four, columns that are not a multiple of eight, operands that
     // start off the 16-byte grid: the instantiation that repairs the last bytes of a and b and stores c
     // without assuming any alignment of its rows
-    const bool tails = (a.lda & 3) != 0 || (a.n & 7) != 0 || (((uintptr_t)a.a | (uintptr_t)a.b | (uintptr_t)a.c) & 15) != 0;
+    // (with the fused epilogue the rows of the output have n/2 columns: 16-byte stores need n/2 on the 8-column grid)
+    const int out_cols = EPI == 1 ? a.n / 2 : a.n;
+    const bool tails = (a.lda & 3) != 0 || (a.n & 7) != 0 || (out_cols & 7) != 0 || (((uintptr_t)a.a | (uintptr_t)a.b | (uintptr_t)a.c) & 15) != 0;
     void (*kern)(const GemmArgs) = tails ? gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI, NSTAGE, true> : gemm_tr_kernel<BM, BN, WM, WN, MODE, EPI, NSTAGE, false>;
     static int raised[2][MAX_DEVICES];
     hipError_t e = raise_lds_limit((const void*)kern, C::LDS_BYTES, raised[tails ? 1 : 0]);

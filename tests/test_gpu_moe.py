@@ -45,7 +45,8 @@ def _within(oracle, out, ref, what):
 
 @pytest.mark.parametrize("m,n,k", [(256, 512, 512), (272, 288, 256), (100, 70, 128), (512, 4096, 1024),
                                    (257, 512, 256), (1023, 288, 384), (3, 64, 128), (130, 4096, 128),      # rows off the 4-row grid
-                                   (300, 380, 256), (129, 2002, 128), (64, 6, 128), (513, 1038, 384)])     # n/2 off the 8-column grid: rows of h stored in pieces
+                                   (300, 380, 256), (129, 2002, 128), (64, 6, 128), (513, 1038, 384),      # n/2 off the 8-column grid: rows of h stored in pieces
+                                   (128, 72, 128), (300, 296, 256), (257, 1080, 384), (64, 8, 128)])       # n on the 8-column grid, n/2 four columns off it
 def test_dense_silu_mul(pkg, moe, oracle, mo, dev, m, n, k):
     """std 0.02 weights keep gate/up at O(1) so that silu is exercised around its bend"""
     g = torch.Generator().manual_seed(m + n)
@@ -59,7 +60,8 @@ def test_dense_silu_mul(pkg, moe, oracle, mo, dev, m, n, k):
 
 
 @pytest.mark.parametrize("tokens,n", [(160, 512), (161, 512), (67, 512),        # 480 rows; 483 and 201: totals off the 4-row grid
-                                      (160, 380), (67, 2002), (161, 262)])      # n/2 off the 8-column grid, n off the 4-byte grid of b's rows
+                                      (160, 380), (67, 2002), (161, 262),       # n/2 off the 8-column grid, n off the 4-byte grid of b's rows
+                                      (160, 104), (161, 1336), (67, 584)])      # n a multiple of 8 but not of 16
 def test_grouped_silu_mul(pkg, moe, oracle, mo, dev, tokens, n):
     cfg = pkg.inputs.CONFIGS[4]
     data = pkg.inputs.make_grouped(cfg, tokens=tokens, n=n, k=256, experts=6, topk=3)
