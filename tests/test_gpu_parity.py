@@ -343,6 +343,30 @@ def test_runs_on_the_current_stream(pkg, oracle, dev):
     _check_mfma(oracle, out, oracle.ref_kernel(cpu), "side stream", cpu, 4)
 
 
+def test_k_splits_that_overlap_on_two_streams(pkg, oracle, dev):
+    """custom_kernel keeps one K-split workspace per device and stream: two different split-K problems issued
+    alternately on two streams, many times and without waiting in between, each give their serial result."""
+    cfg = pkg.inputs.CONFIGS[3]
+    probs = []
+    for (m, n, k), seed in (((64, 2304, 2048), 3), ((48, 4608, 4096), 4)):
+        assert pkg.plan(m, n, k).split_k > 1
+        data = _to(pkg.inputs.make_dense(pkg.inputs.Config("two streams", m, n, k, cfg.a_outlier_frac, cfg.a_outlier_mul, cfg.b_std, 0, 0, seed)), dev)
+        serial = pkg.custom_kernel(tuple(data[:4]) + (torch.empty_like(data[4]),)).clone()
+        probs.append((data, serial))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[], []]
+    for rep in range(20):
+        for i, (data, _) in enumerate(probs):
+            with torch.cuda.stream(streams[i]):
+                c = torch.empty_like(data[4])
+                outs[i].append(pkg.custom_kernel(tuple(data[:4]) + (c,)))
+    torch.cuda.synchronize()
+    for i, (_, serial) in enumerate(probs):
+        for rep, c in enumerate(outs[i]):
+            assert torch.equal(c.view(torch.int16), serial.view(torch.int16)), "stream %d call %d" % (i, rep)
+
+
 @pytest.mark.parametrize("idx", [1, 2, 3])
 def test_full_size_dense_configs(pkg, oracle, dev, idx):
     """Configurations 2-4 at their published sizes against the oracle on every element."""

@@ -63,3 +63,36 @@ def test_without_a_split_and_beyond_the_limit(pkg, dev):
     torch.cuda.synchronize()
     assert st == 8 and b"scratch" in lib.fp8bs_strerror(st)
     assert bool((c == 7.0).all())
+
+
+def test_under_graph_capture(pkg, dev):
+    """what the entry point is for: a call with a K split captured into a HIP graph (no allocation, no workspace
+    argument) and replayed with other inputs, eager work and synchronisation in between - every replay equals the
+    eager result of fp8bs_gemm bit for bit"""
+    lib = pkg._lib.load()
+    cfg = pkg.inputs.CONFIGS[3]
+    m, n, k = 64, 2304, 2048
+    assert pkg.plan(m, n, k).split_k > 1
+    sets = [tuple(t.to(dev) for t in pkg.inputs.make_dense(pkg.inputs.Config("capture", m, n, k, cfg.a_outlier_frac, cfg.a_outlier_mul, cfg.b_std, 0, 0, s)))
+            for s in (1, 2)]
+    eager = [pkg.custom_kernel(tuple(s[:4]) + (torch.empty_like(s[4]),)).clone() for s in sets]
+    static = tuple(t.clone() for t in sets[0])
+
+    def call():
+        pkg._lib.check(lib.fp8bs_gemm_noalloc(static[0].data_ptr(), static[1].data_ptr(), static[2].data_ptr(), static[3].data_ptr(),
+                                              static[4].data_ptr(), m, n, k, torch.cuda.current_stream().cuda_stream))
+    call()                                                        # outside capture: the array's address is looked up here
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for rep in range(4):
+        src, want = sets[rep % 2], eager[rep % 2]
+        for dst, s in zip(static[:4], src[:4]):
+            dst.copy_(s)
+        static[4].fill_(3.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static[4].view(torch.int16), want.view(torch.int16)), "replay %d" % rep
+        pkg.custom_kernel(sets[(rep + 1) % 2])                    # eager work between replays
+        torch.cuda.synchronize()
