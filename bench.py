@@ -186,7 +186,8 @@ def mfma_ceiling(pkg, dev):
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     names = {0: "mfma", 1: "mfma+fold", 2: "mfma+lds_reads", 3: "mfma+fold+lds_reads", 4: "mfma+copies", 5: "mfma+fold+copies",
              6: "mfma+lds_reads+copies", 7: "mfma+fold+lds_reads+copies", 8: "mfma32x32x64", 9: "mfma32x32x64+fold",
-             11: "mfma32x32x64+fold+lds_reads", 15: "mfma32x32x64+fold+lds_reads+copies"}
+             11: "mfma32x32x64+fold+lds_reads", 15: "mfma32x32x64+fold+lds_reads+copies",
+             19: "mfma+fold+lds_reads(spread evenly)", 23: "mfma+fold+lds_reads(spread evenly)+copies"}
     iters = 1500                                                                  # 1500 x 2048 clk = 1.28 ms at 2.4 GHz
     rows = []
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -228,10 +228,12 @@ int fp8bs_moe_combine(const void* y, int rows, const int32_t* slot_of, const flo
 /* ---- Measurement aid -------------------------------------------------------------------------------
  * No counterpart in the reference and no part of any GEMM call: runs, `iters` times per wave, the
  * instruction mix of one K block of the 256x256 tile's wave (32 FP8 MFMAs on random operands, 8 waves per
- * workgroup) with the parts selected by the bits of `mix` (0 .. 15): 1 = the scale fold (4 v_fma per MFMA),
+ * workgroup) with the parts selected by the bits of `mix` (0 .. 23): 1 = the scale fold (4 v_fma per MFMA),
  * 2 = the transposing LDS reads (48 per 32 MFMAs), 4 = the global->LDS copies (8 KiB per wave per 32 MFMAs;
  * the 8 workgroups an XCD runs side by side share a stream, the streams walk src cyclically), 8 = the same
- * multiply-accumulates as 16 MFMAs of the 32x32x64 form - without barriers, waits or output.  One iteration is 2048 clocks of matrix-core work per SIMD, so
+ * multiply-accumulates as 16 MFMAs of the 32x32x64 form, 16 (with bit 2 only) = the LDS reads spread evenly
+ * over the K block into a second set of A registers instead of the GEMM's bursts - without barriers, waits or
+ * output; `iters` must be even (the loop body is two K blocks, one per LDS stage, all LDS addresses immediate).  One iteration is 2048 clocks of matrix-core work per SIMD, so
  * iters * 2048 / 2.4e9 / time is the fraction of the nominal FP8 peak the mix reaches on `workgroups` CUs.
  * src: device buffer of src_bytes (a power of two >= 4 MiB, 16-byte aligned) whose first 64 KiB hold e4m3fn
  * codes used as operands; sink: 4 writable device bytes (never written in practice).  bench.py
