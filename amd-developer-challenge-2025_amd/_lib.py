@@ -88,6 +88,29 @@ def load() -> ctypes.CDLL:
     return lib
 
 
+_pycall = False
+
+
+def pycall():
+    """The CPython binding of fp8bs_gemm_ex / fp8bs_gemm_grouped_ex (csrc/fp8bs_pycall.c: the same library
+    functions without ctypes' per-argument marshalling), or None where it has not been built; callers then use
+    the ctypes functions of load().  Either way the work is done by libfp8bs.so, which has no substitute."""
+    global _pycall
+    if _pycall is False:
+        load()                                        # the library must be there first; raises if it is not
+        path = os.path.join(HERE, "_fp8bs_pycall.so")
+        _pycall = None
+        if os.path.exists(path):
+            import importlib.machinery
+            import importlib.util
+            loader = importlib.machinery.ExtensionFileLoader("_fp8bs_pycall", path)
+            spec = importlib.util.spec_from_file_location("_fp8bs_pycall", path, loader=loader)
+            mod = importlib.util.module_from_spec(spec)
+            loader.exec_module(mod)
+            _pycall = mod
+    return _pycall
+
+
 def check(status: int) -> None:
     """Raise RuntimeError with the library's message for a non-zero status."""
     if status != 0:

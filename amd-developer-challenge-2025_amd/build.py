@@ -11,6 +11,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 LIB_PATH = os.path.join(HERE, "libfp8bs.so")
+PYCALL_PATH = os.path.join(HERE, "_fp8bs_pycall.so")
 CSRC = os.path.join(HERE, "csrc")
 SOURCES = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 OBJ_DIR = os.path.join(HERE, "csrc", "_obj")          # git-ignored build products
@@ -49,7 +50,22 @@ def build(verbose: bool = False, jobs: int = 0) -> str:
     if rc != 0:
         sys.stderr.write(out)
         raise RuntimeError("hipcc failed linking libfp8bs.so (exit %d)" % rc)
+    build_pycall(verbose)
     return LIB_PATH
+
+
+def build_pycall(verbose: bool = False) -> str:
+    """The CPython binding of the two GEMM entry points (csrc/fp8bs_pycall.c): host compiler, linked against
+    libfp8bs.so next to it.  Replaces ctypes' argument marshalling on the hot call path only."""
+    import sysconfig
+    cc = os.environ.get("CC", "gcc")
+    cmd = [cc, "-O2", "-shared", "-fPIC", "-I" + sysconfig.get_paths()["include"], "-I" + os.path.join(ROOT, "include"),
+           "-o", PYCALL_PATH, os.path.join(CSRC, "fp8bs_pycall.c"), "-L" + HERE, "-lfp8bs", "-Wl,-rpath,$ORIGIN"]
+    rc, out = _run(cmd, verbose)
+    if rc != 0:
+        sys.stderr.write(out)
+        raise RuntimeError("%s failed building _fp8bs_pycall.so (exit %d)" % (cc, rc))
+    return PYCALL_PATH
 
 
 if __name__ == "__main__":

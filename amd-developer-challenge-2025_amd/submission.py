@@ -50,26 +50,41 @@ def _is_kmajor(t: torch.Tensor) -> bool:
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 _plan_cache = {}   # (m, n, k) -> workspace bytes the planner asks for
 
-# Operands that passed the checks once: a caller that hands over the same five tensor objects again
-# (a benchmark loop, a layer called every step) skips the dtype / device / K-major checks, which cost more
-# host time than a small GEMM takes on the GPU.  An entry is keyed by the identities and version counters
-# of the tensors and holds weak references, so a recycled id() cannot alias a dead tensor; what the
-# version counter does not cover (resize_, set_, .data = ...) is caught by comparing the addresses, shapes
-# and strides kept with the entry.  Tensors without a version counter (made under inference_mode) take
-# the full checks every time.
+# Operands that passed the checks once: a caller that hands over the same tensor objects again (a benchmark
+# loop, a layer called every step) skips the dtype / device / K-major checks, which cost more host time than a
+# small GEMM takes on the GPU.  An entry is keyed by the identities of the tensors and holds weak references,
+# so a recycled id() cannot alias a dead tensor; what can change under one identity (resize_, set_, as_strided_,
+# t_, .data = ...) is caught by comparing addresses, shapes and strides with the ones that were checked.
 _CHECKED_MAX = 64
-_checked = {}      # key -> (weakrefs, (addresses, shapes, strides), m, n, k, workspace bytes, device index)
+_checked = {}      # ids -> (weakrefs, addresses, shapes, strides, sizes ..., device index)
 
 
-def _cache_key(ts):
-    try:
-        return tuple(x for t in ts for x in (id(t), t._version))
-    except RuntimeError:
-        return None
+def _remember(key, data, *rest):
+    if len(_checked) >= _CHECKED_MAX:
+        _checked.pop(next(iter(_checked)))
+    _checked[key] = (tuple(weakref.ref(t) for t in data), tuple(t.data_ptr() for t in data), tuple(t.shape for t in data),
+                     tuple(t.stride() for t in data)) + rest
 
 
-def _layout(ts):
-    return tuple(t.data_ptr() for t in ts), tuple(t.shape for t in ts), tuple(t.stride() for t in ts)
+def _gemm_ex_fn():
+    """fp8bs_gemm_ex through the CPython binding when it is built, else through ctypes (same library function)."""
+    fast = _lib.pycall()
+    return fast.gemm_ex if fast is not None else _lib.load().fp8bs_gemm_ex
+
+
+def _grouped_ex_fn():
+    fast = _lib.pycall()
+    return fast.gemm_grouped_ex if fast is not None else _lib.load().fp8bs_gemm_grouped_ex
+
+
+_gemm_ex = _grouped_ex = None
+
+
+def _bind():
+    """Resolve the two call targets once (the CPython binding if built, else ctypes)."""
+    global _gemm_ex, _grouped_ex
+    _gemm_ex, _grouped_ex = _gemm_ex_fn(), _grouped_ex_fn()
+    return _gemm_ex, _grouped_ex
 
 
 def _stream_ptr(device: torch.device) -> int:
@@ -119,22 +134,27 @@ def custom_kernel(data, variant: int = 0, split_k: int = 0):
     the defaults let the library's planner decide.
     """
     a, b, a_scale, b_scale, c = data
-    lib = _lib.load()
-    key = _cache_key(data) if variant == 0 and split_k == 0 else None
-    if key is not None:
+    gemm_ex = _gemm_ex or _bind()[0]
+    key = None
+    if variant == 0 and split_k == 0:
+        key = (id(a), id(b), id(a_scale), id(b_scale), id(c))
         hit = _checked.get(key)
         if hit is not None:
-            refs, layout, m, n, k, need, dev_index = hit
-            now = _layout(data)
+            refs, ptrs, shapes, strides, m, n, k, need, dev_index = hit
+            pa, pb, pas, pbs, pc = a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(), c.data_ptr()
             if refs[0]() is a and refs[1]() is b and refs[2]() is a_scale and refs[3]() is b_scale and refs[4]() is c \
-                    and now == layout and dev_index == torch.cuda.current_device():
+                    and (pa, pb, pas, pbs, pc) == ptrs \
+                    and a.shape == shapes[0] and b.shape == shapes[1] and a_scale.shape == shapes[2] and b_scale.shape == shapes[3] and c.shape == shapes[4] \
+                    and a.stride() == strides[0] and b.stride() == strides[1] and a_scale.stride() == strides[2] \
+                    and b_scale.stride() == strides[3] and c.stride() == strides[4] and dev_index == torch.cuda.current_device():
                 stream = _stream_ptr(a.device)
                 ws_ptr, ws_len = None, 0
                 if need:
                     ws = _workspace(a.device, need, stream)
                     ws_ptr, ws_len = ws.data_ptr(), ws.numel()
-                ptrs = now[0]
-                _lib.check(lib.fp8bs_gemm_ex(ptrs[0], ptrs[1], ptrs[2], ptrs[3], ptrs[4], ws_ptr, ws_len, m, n, k, 0, 0, stream))
+                st = gemm_ex(pa, pb, pas, pbs, pc, ws_ptr, ws_len, m, n, k, 0, 0, stream)
+                if st:
+                    _lib.check(st)
                 return c
     m, k = a.shape
     n = b.shape[0]
@@ -149,10 +169,7 @@ def custom_kernel(data, variant: int = 0, split_k: int = 0):
         if need is None:
             need = workspace_bytes(m, n, k) if (m > 0 and n > 0 and k > 0) else 0
             _plan_cache[(m, n, k)] = need
-        if key is not None:
-            if len(_checked) >= _CHECKED_MAX:
-                _checked.pop(next(iter(_checked)))
-            _checked[key] = (tuple(weakref.ref(t) for t in data), _layout(data), m, n, k, need, a.device.index)
+        _remember(key, data, m, n, k, need, a.device.index)
     else:
         need = max(split_k, 1) * m * n * 4 if split_k > 1 else 0
     # kernels are launched on the device the pointers live on: the library uses the current device
@@ -162,8 +179,8 @@ def custom_kernel(data, variant: int = 0, split_k: int = 0):
         if need:
             ws = _workspace(a.device, need, stream)
             ws_ptr, ws_len = ws.data_ptr(), ws.numel()
-        st = lib.fp8bs_gemm_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
-                               c.data_ptr(), ws_ptr, ws_len, m, n, k, variant, split_k, stream)
+        st = gemm_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
+                     c.data_ptr(), ws_ptr, ws_len, m, n, k, variant, split_k, stream)
     _lib.check(st)
     return c
 
@@ -179,19 +196,18 @@ def grouped_kernel(data, variant: int = 0):
     [E, ceil(n/128), k/128] with stride (nb*kb, 1, nb).  Fills and returns ``c``; no host sync.
     """
     a, b, a_scale, b_scale, row_offsets, c = data
-    lib = _lib.load()
-    key = _cache_key(data)
-    if key is not None:
-        key = ("grouped",) + key
-        hit = _checked.get(key)
-        if hit is not None:
-            refs, layout, rows, n, k, num_experts, dev_index = hit
-            now = _layout(data)
-            if all(r() is t for r, t in zip(refs, data)) and now == layout and dev_index == torch.cuda.current_device():
-                ptrs = now[0]
-                _lib.check(lib.fp8bs_gemm_grouped_ex(ptrs[0], ptrs[1], ptrs[2], ptrs[3], ptrs[5], ptrs[4], num_experts, rows, n, k,
-                                                     variant, _stream_ptr(a.device)))
-                return c
+    grouped_ex = _grouped_ex or _bind()[1]
+    key = ("grouped", id(a), id(b), id(a_scale), id(b_scale), id(row_offsets), id(c))
+    hit = _checked.get(key)
+    if hit is not None:
+        refs, ptrs, shapes, strides, rows, n, k, num_experts, dev_index = hit
+        now = tuple(t.data_ptr() for t in data)
+        if all(r() is t for r, t in zip(refs, data)) and now == ptrs and tuple(t.shape for t in data) == shapes \
+                and tuple(t.stride() for t in data) == strides and dev_index == torch.cuda.current_device():
+            st = grouped_ex(now[0], now[1], now[2], now[3], now[5], now[4], num_experts, rows, n, k, variant, _stream_ptr(a.device))
+            if st:
+                _lib.check(st)
+            return c
     rows, k = a.shape
     if b.dim() != 3:
         raise ValueError("b must be [E, n, k]")
@@ -204,12 +220,9 @@ def grouped_kernel(data, variant: int = 0):
         raise ValueError("every expert of b and b_scale must be K-major")
     if row_offsets.dtype != torch.int32 or tuple(row_offsets.shape) != (num_experts + 1,) or row_offsets.device != a.device:
         raise ValueError("row_offsets must be an int32 tensor with num_experts+1 entries on the operands' GPU")
-    if key is not None:
-        if len(_checked) >= _CHECKED_MAX:
-            _checked.pop(next(iter(_checked)))
-        _checked[key] = (tuple(weakref.ref(t) for t in data), _layout(data), rows, n, k, num_experts, a.device.index)
+    _remember(key, data, rows, n, k, num_experts, a.device.index)
     with torch.cuda.device(a.device):
-        st = lib.fp8bs_gemm_grouped_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
-                                       c.data_ptr(), row_offsets.data_ptr(), num_experts, rows, n, k, variant, _stream_ptr(a.device))
+        st = grouped_ex(a.data_ptr(), b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(),
+                        c.data_ptr(), row_offsets.data_ptr(), num_experts, rows, n, k, variant, _stream_ptr(a.device))
     _lib.check(st)
     return c

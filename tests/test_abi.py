@@ -148,6 +148,30 @@ def test_custom_kernel_without_version_counters(pkg):
             pkg.custom_kernel(data)
 
 
+def test_cpython_binding_returns_what_ctypes_returns(pkg):
+    """csrc/fp8bs_pycall.c binds fp8bs_gemm_ex / fp8bs_gemm_grouped_ex without ctypes' marshalling: built by build(),
+    same status codes for the argument errors that are reported before any launch, type errors raised."""
+    lib, fast = pkg._lib.load(), pkg._lib.pycall()
+    assert fast is not None, "the CPython binding was not built (amd-developer-challenge-2025_amd/build.py)"
+    one = 16
+    for args in ((one, one, one, one, one, None, 0, 16, 16, 100, 0, 0, None),          # k not a multiple of 128
+                 (None, one, one, one, one, None, 0, 16, 16, 128, 0, 0, None),         # null pointer
+                 (one, one, one, one, one, None, 0, 0, 16, 128, 0, 0, None),           # empty
+                 (one, one, one, one, one, None, 0, 1 << 20, 16, 1 << 13, 0, 0, None), # too large
+                 (one, one, one, one, one, None, 0, 16, 16, 128, 99, 1, None),         # unknown variant
+                 (one, one, one, one, one, None, 0, 64, 256, 1024, 4, 4, None)):       # forced K split without a workspace
+        assert fast.gemm_ex(*args) == lib.fp8bs_gemm_ex(*args)
+    g = (one, one, one, one, one, None, 4, 16, 16, 128, 0, None)
+    assert fast.gemm_grouped_ex(*g) == lib.fp8bs_gemm_grouped(*(g[:10] + g[11:])) == 1
+    assert fast.gemm_grouped_ex(one, one, one, one, one, one, 0, 16, 16, 128, 0, None) == 6
+    with pytest.raises(TypeError):
+        fast.gemm_ex(1, 2, 3)
+    with pytest.raises(TypeError):
+        fast.gemm_ex("a", one, one, one, one, None, 0, 16, 16, 128, 0, 0, None)
+    with pytest.raises(OverflowError):
+        fast.gemm_ex(one, one, one, one, one, None, 0, 1 << 40, 16, 128, 0, 0, None)
+
+
 def test_root_submission_module_reexports_entry_point(pkg):
     import submission
     assert submission.custom_kernel is pkg.custom_kernel

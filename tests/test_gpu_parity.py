@@ -133,8 +133,8 @@ def test_many_tiles_per_workgroup_against_the_scalar_kernel(pkg, oracle, dev, m,
 
 
 def test_repeated_calls_skip_the_checks_but_not_after_a_change(pkg, oracle, dev):
-    """The second call with the same tensor objects takes the short path; a tensor changed in place, or
-    another tensor object of a wrong layout, is checked again."""
+    """The second call with the same tensor objects takes the short path; a tensor whose layout was changed in
+    place (strides, shape), or another tensor object of a wrong layout, is checked again."""
     sub = importlib.import_module("amd-developer-challenge-2025_amd.submission")
     cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[2], m=64, n=256, k=256)
     ref = oracle.ref_kernel(cpu)
@@ -142,16 +142,21 @@ def test_repeated_calls_skip_the_checks_but_not_after_a_change(pkg, oracle, dev)
     sub._checked.clear()
     out1 = pkg.custom_kernel((a, b, a_scale, b_scale, c)).clone()
     assert len(sub._checked) == 1
-    c.zero_()                                                   # bumps c's version: a new entry, same answer
+    c.zero_()                                                   # new contents, same layout: the short path, same answer
     out2 = pkg.custom_kernel((a, b, a_scale, b_scale, c)).clone()
-    out3 = pkg.custom_kernel((a, b, a_scale, b_scale, c))     # the short path
-    assert out3 is c and len(sub._checked) == 2
+    out3 = pkg.custom_kernel((a, b, a_scale, b_scale, c))
+    assert out3 is c and len(sub._checked) == 1
     for o in (out1, out2, out3):
         _check(oracle, o, ref, "repeated call")
     a_scale.transpose_(0, 1)                                    # same object, now [k/128, m]: must be refused
     with pytest.raises(ValueError):
         pkg.custom_kernel((a, b, a_scale, b_scale, c))
     a_scale.transpose_(0, 1)
+    c.resize_(32, 256)                                          # same object and address, half the rows: must be refused
+    with pytest.raises(ValueError):
+        pkg.custom_kernel((a, b, a_scale, b_scale, c))
+    c.resize_(64, 256)
+    _check(oracle, pkg.custom_kernel((a, b, a_scale, b_scale, c)), ref, "after the layout was restored")
     with pytest.raises(ValueError):
         pkg.custom_kernel((a, b, a_scale.contiguous(), b_scale, c))    # row-major copy: wrong strides
     del a, b, a_scale, b_scale, c, out3
