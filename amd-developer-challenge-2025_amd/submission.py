@@ -32,6 +32,8 @@ def _workspace(device: torch.device, nbytes: int, stream: int = 0) -> torch.Tens
     key = (device.index, stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if ws is None and len(_workspaces) >= 16:     # streams come and go: keep the table bounded (oldest entry out)
+            _workspaces.pop(next(iter(_workspaces)))
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
