@@ -46,7 +46,7 @@ enum {
 /* Kernel variants the planner chooses from. */
 enum {
     FP8BS_VARIANT_AUTO = 0,
-    FP8BS_VARIANT_GENERIC = 1,    /* scalar kernel, any m/n (alignment fallback)             */
+    FP8BS_VARIANT_GENERIC = 1,    /* scalar kernel, any m/n: the planner uses it for k = 0 only */
     FP8BS_VARIANT_T256x256 = 2,   /* compute-bound: 256x256 tile, 8 waves                    */
     FP8BS_VARIANT_T128x128 = 3,   /* mid-size: 128x128 tile, 4 waves                         */
     FP8BS_VARIANT_T64x128 = 4,    /* skinny-M: 64(m) x 128(n) tile, 4 waves, split-K         */
