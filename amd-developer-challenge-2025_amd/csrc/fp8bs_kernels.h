@@ -23,6 +23,7 @@ struct GemmArgs {
     int band_h;             // tile rows per band of the tile walk
     int num_experts;
     int epi;                // 0: bf16 of the product; 1: silu(column 2i) * column 2i+1, n/2 output columns
+    int c_whole_lines;      // set by the launcher: rows of c start and end on 128-byte lines
 };
 
 // Per-device bookkeeping of the launchers.  A kernel's dynamic-LDS limit is a property of the kernel
