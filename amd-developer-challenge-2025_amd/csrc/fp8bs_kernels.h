@@ -24,6 +24,7 @@ struct GemmArgs {
     int num_experts;
     int epi;                // 0: bf16 of the product; 1: silu(column 2i) * column 2i+1, n/2 output columns
     int c_whole_lines;      // set by the launcher: rows of c start and end on 128-byte lines
+    int by_expert;          // grouped: order of the tiles, 0 across the experts, 1 expert by expert (see the tile walk)
 };
 
 // Per-device bookkeeping of the launchers.  A kernel's dynamic-LDS limit is a property of the kernel

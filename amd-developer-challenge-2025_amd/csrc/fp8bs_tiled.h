@@ -47,6 +47,7 @@ typedef unsigned short v4us __attribute__((ext_vector_type(4)));
 #define LDS_VOID(p) ((__attribute__((address_space(3))) void*)(p))
 
 static constexpr int KBLK = 128;  // scale block along K == K extent of one MFMA
+static constexpr int GROUP_TABLE_MAX = 128;   // grouped walk: up to 127 experts have their row ranges kept in LDS (2 KiB)
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     v2f f = {lo, hi};
@@ -250,12 +251,48 @@ void gemm_tr_kernel(const GemmArgs p) {
         const float* bsptr;
     };
     int total_slots = 0;                      // grouped: m-tile slots that exist (from row_offsets)
-    if (MODE == 2)
-        for (int x = 0; x < p.num_experts; x++) {
-            int lo = p.row_offsets[x], hi = p.row_offsets[x + 1];
-            lo = lo < 0 ? 0 : lo; hi = hi > p.m ? p.m : hi;       // a malformed table must not reach beyond the matrix
-            total_slots += (hi > lo) ? (hi - (lo & ~15) + BM - 1) / BM : 0;
+    // Grouped, fewer than GROUP_TABLE_MAX experts: a table in LDS, one entry per expert - first row of its first
+    // tile (row_offsets[e] rounded down to 16), its row range, and the number of slots before it - built once
+    // by wave 0.  Finding a tile's expert is then one LDS read per lane and a count of the lanes whose experts
+    // start at or before the tile's slot; as a loop over row_offsets in scalar code it took 1.5-2 us per tile,
+    // between the last K block of one tile and the first copies of the next.  More experts: that loop.
+    [[maybe_unused]] v4i* gtable = nullptr;
+    bool use_table = false;
+    if constexpr (MODE == 2) {
+        __shared__ v4i gtable_store[GROUP_TABLE_MAX];        // entry [num_experts]: the slots before the end = all of them
+        gtable = gtable_store;
+        use_table = p.num_experts < GROUP_TABLE_MAX;
+        if (use_table) {
+            if (wave == 0) {
+                int carry = 0;
+                for (int base = 0; base < p.num_experts; base += 64) {
+                    const int x = base + lane;
+                    int lo = 0, hi = 0;
+                    if (x < p.num_experts) { lo = p.row_offsets[x]; hi = p.row_offsets[x + 1]; }
+                    lo = lo < 0 ? 0 : lo; hi = hi > p.m ? p.m : hi;       // a malformed table must not reach beyond the matrix
+                    const int s = lo & ~15;
+                    const int nt = (hi > lo) ? (hi - s + BM - 1) / BM : 0;
+                    int incl = nt;                                        // inclusive prefix sum over the 64 lanes
+#pragma unroll
+                    for (int d = 1; d < 64; d <<= 1) {
+                        const int y = __shfl_up(incl, d, 64);
+                        if (lane >= d) incl += y;
+                    }
+                    if (x < p.num_experts) gtable_store[x] = (v4i){s, lo, hi, carry + incl - nt};
+                    carry += __shfl(incl, 63, 64);
+                }
+                if (lane == 0) gtable_store[p.num_experts] = (v4i){0, 0, 0, carry};
+            }
+            __syncthreads();
+            total_slots = __builtin_amdgcn_readfirstlane(gtable_store[p.num_experts][3]);
+        } else {
+            for (int x = 0; x < p.num_experts; x++) {
+                int lo = p.row_offsets[x], hi = p.row_offsets[x + 1];
+                lo = lo < 0 ? 0 : lo; hi = hi > p.m ? p.m : hi;
+                total_slots += (hi > lo) ? (hi - (lo & ~15) + BM - 1) / BM : 0;
+            }
         }
+    }
     auto pick_tile = [&](int it) -> Tile {
         Tile t;
         t.valid = 0; t.m0 = 0; t.n0 = 0; t.kb_begin = 0; t.kb_end = 0; t.split_z = 0; t.row_lo = 0; t.row_hi = p.m;
@@ -265,26 +302,56 @@ void gemm_tr_kernel(const GemmArgs p) {
             // grouped: m-tile slots are laid over the experts in order; expert e's tiles start at
             // row_offsets[e] rounded down to 16 so that global 16-byte loads stay aligned; rows outside
             // [row_offsets[e], row_offsets[e+1]) are computed but never stored.  The gridDim.x tiles in
-            // flight together are dealt to the XCDs in contiguous runs and laid over the (slot, n tile)
-            // grid in bands of band_h slots, as in the dense case, so that the tiles sharing an L2 form a
-            // compact block of few A panels and few B panels.
+            // flight together are dealt to the XCDs in contiguous runs.  Two orders of the tiles.  Across
+            // the experts: the (slot, n tile) grid of all slots in bands of band_h slots, as in the dense case.
+            // Expert by expert (p.by_expert): inside an expert's own grid in bands, an expert of up to eight
+            // slots being one band, so that the tiles sharing an L2 form a compact block of few A panels and
+            // few B panels of one expert and the tile that holds an expert's last rows runs beside the full
+            // tiles that read the same panel of the expert's weights.
             const int tiles_n = (p.n + BN - 1) / BN;
             const int total = total_slots * tiles_n;
             const int v = it * G + xcd_virtual_id(blockIdx.x, G);
             if (v >= total) return t;
-            int slot, tn;
-            band_tile(v, total_slots, tiles_n, p.band_h, slot, tn);
+            const bool by_expert = p.by_expert != 0;
+            int slot_all = 0, tn = 0;
+            if (!by_expert) band_tile(v, total_slots, tiles_n, p.band_h, slot_all, tn);
             int e = 0, found = 0, start = 0, cnt_lo = 0, cnt_hi = 0;
-            int acc_tiles = 0;
-            for (int x = 0; x < p.num_experts; x++) {
-                int lo = p.row_offsets[x], hi = p.row_offsets[x + 1];
-                lo = lo < 0 ? 0 : lo; hi = hi > p.m ? p.m : hi;
-                int s = lo & ~15;
-                int nt = (hi > lo) ? (hi - s + BM - 1) / BM : 0;
-                if (!found && slot < acc_tiles + nt) {
-                    found = 1; e = x; start = s + (slot - acc_tiles) * BM; cnt_lo = lo; cnt_hi = hi;
+            if (use_table) {
+                // the expert whose slots hold slot `key`: the last one that starts at or before it (experts
+                // without rows start where the next one starts, and are never the last such)
+                const int key = by_expert ? v / tiles_n : slot_all;
+                int cnt = 0;
+                for (int base = 0; base < p.num_experts; base += 64) {
+                    const int x = base + lane;
+                    const int before = x < p.num_experts ? gtable[x][3] : 0x7FFFFFFF;
+                    cnt += __popcll(__ballot(before <= key));
                 }
-                acc_tiles += nt;
+                cnt = __builtin_amdgcn_readfirstlane(cnt);
+                if (cnt > 0) {
+                    e = cnt - 1;
+                    const v4i row = gtable[e];
+                    const int s = __builtin_amdgcn_readfirstlane(row[0]), before = __builtin_amdgcn_readfirstlane(row[3]);
+                    cnt_lo = __builtin_amdgcn_readfirstlane(row[1]); cnt_hi = __builtin_amdgcn_readfirstlane(row[2]);
+                    const int nt = (cnt_hi > cnt_lo) ? (cnt_hi - s + BM - 1) / BM : 0;
+                    int slot = slot_all - before;
+                    if (by_expert) band_tile(v - before * tiles_n, nt, tiles_n, nt <= 8 ? nt : p.band_h, slot, tn);
+                    found = slot < nt;
+                    start = s + slot * BM;
+                }
+            } else {
+                int acc_slots = 0;
+                for (int x = 0; x < p.num_experts; x++) {
+                    int lo = p.row_offsets[x], hi = p.row_offsets[x + 1];
+                    lo = lo < 0 ? 0 : lo; hi = hi > p.m ? p.m : hi;
+                    int s = lo & ~15;
+                    int nt = (hi > lo) ? (hi - s + BM - 1) / BM : 0;
+                    if (!found && (by_expert ? v < (acc_slots + nt) * tiles_n : slot_all < acc_slots + nt)) {
+                        int slot = slot_all - acc_slots;
+                        if (by_expert) band_tile(v - acc_slots * tiles_n, nt, tiles_n, nt <= 8 ? nt : p.band_h, slot, tn);
+                        found = 1; e = x; start = s + slot * BM; cnt_lo = lo; cnt_hi = hi;
+                    }
+                    acc_slots += nt;
+                }
             }
             if (!found) return t;                      // uniform for the whole workgroup
             t.valid = 1;
@@ -878,7 +945,7 @@ static inline hipError_t launch_shape(const GemmArgs& a, int mode, hipStream_t s
     using C = TileCfg<BM, BN, WM, WN, 0, NSTAGE>;
     // persistent workgroups: as many as fit the chip at once (LDS and thread limits), each walks
     // tiles  blockIdx.x, blockIdx.x + grid, ...
-    const int by_lds = 163840 / C::LDS_BYTES, by_threads = 2048 / C::NTHREADS;
+    const int by_lds = 163840 / (C::LDS_BYTES + (mode == 2 ? GROUP_TABLE_MAX * 16 : 0)), by_threads = 2048 / C::NTHREADS;   // (grouped: + the table of the experts)
     const long resident = (long)device_cus() * (by_lds < by_threads ? by_lds : by_threads);
     const int tiles_n = (a.n + BN - 1) / BN;
     long total;

@@ -401,6 +401,24 @@ def test_grouped_small(pkg, oracle, dev, tokens, n, k, experts, topk):
     _check(oracle, out, oracle.ref_grouped(cpu), "grouped %s" % ((tokens, n, k, experts, topk),))
 
 
+@pytest.mark.parametrize("variant", [0, 3, 11])
+@pytest.mark.parametrize("tokens,n,k,experts,topk", [(200, 256, 256, 70, 3), (500, 136, 128, 127, 2), (500, 136, 128, 128, 2),
+                                                      (300, 256, 128, 200, 4), (2048, 512, 256, 3, 2), (6000, 256, 128, 2, 1),
+                                                      (3000, 384, 128, 9, 1)])
+def test_grouped_expert_counts_and_tile_orders(pkg, oracle, dev, variant, tokens, n, k, experts, topk):
+    """The walk's two ways of finding a tile's expert - the table in LDS (fewer than 128 experts; more than 64
+    take two rounds of it) and the loop over row_offsets - and its two orders of the tiles (across the experts
+    when they hold less than a tile of rows on average, expert by expert otherwise, experts of more than eight
+    tile rows cut into bands): every element against the oracle, no row left unwritten."""
+    cpu = pkg.inputs.make_grouped(pkg.inputs.CONFIGS[4], tokens=tokens, n=n, k=k, experts=experts, topk=topk)
+    data = _to(cpu, dev)
+    data[5].fill_(float("nan"))
+    out = pkg.grouped_kernel(data, variant=variant)
+    torch.cuda.synchronize()
+    assert not bool(out.isnan().any())
+    _check(oracle, out, oracle.ref_grouped(cpu), "grouped %s variant %d" % ((tokens, n, k, experts, topk), variant))
+
+
 def test_grouped_full_size_every_element(pkg, oracle, dev):
     """Configuration 5 at its published size (32 experts, 32768 routed rows, N=4096, K=7168): every one of the
     134 million outputs against the oracle (looped per expert on the host cores), and no row left unwritten
