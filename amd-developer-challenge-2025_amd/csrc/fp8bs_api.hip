@@ -31,6 +31,7 @@ bool variant_info(int variant, VariantInfo* out) {
         case FP8BS_VARIANT_T256x192: *out = {256, 192, 512}; return true;
         case FP8BS_VARIANT_T256x128S3: *out = {256, 128, 512}; return true;
         case FP8BS_VARIANT_T192x192S3: *out = {192, 192, 512}; return true;
+        case FP8BS_VARIANT_T64x256S3: *out = {64, 256, 512}; return true;
         default: return false;
     }
 }
@@ -60,18 +61,14 @@ void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out)
     out->workspace_bytes = split_k > 1 ? (uint64_t)split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
 }
 
-// Rows of c (n bf16) that keep 16-byte stores aligned: what the streaming kernels need.  The tiled kernels
-// take any m and n in every mode (they repair the last bytes of a and b themselves, store a row's last chunk
-// of c in pieces, write the partial planes of a K split element by element where rows do not end on a
-// group of four); the streaming kernels take any m.
+// Rows of c (n bf16) that keep 16-byte stores aligned: what the streaming kernels need (forced variants only;
+// the tiled kernels take any m and n in every mode: they repair the last bytes of a and b themselves, store a
+// row's last chunk of c in pieces and write the partial planes of a K split element by element where rows do not
+// end on a group of four).
 bool vector_shape(int n) { return (n % 8) == 0; }
 
-// The streaming kernel is kept for what it was built for: at most 64 rows against a B too large for the
-// caches (configuration 4: 132 MB).  Measured over m = 32 .. 128, n = 512 .. 18432, k = 2048 / 7168 the
-// tiled kernels with a K split are level with it there (38 us either way on configuration 4) and ahead
-// everywhere else: by 3-10 % on smaller B, by 25-30 % from 65 rows on, where the streaming kernel needs a
-// second row of tiles and reads B twice.
-bool streaming_shape(int m, int n, int k) { return m <= 64 && (double)n * (double)k >= 96.0e6; }
+// At most 64 rows against a b of 24 MB or more: the call streams b from HBM once and everything else is small.
+bool skinny_shape(int m, int n, int k) { return m <= 64 && (double)n * (double)k >= 24.0e6; }
 
 // The tile shape and K split of the tiled MFMA kernel that finish soonest (any m, any n).
 void choose_tiled(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may_split = true) {
@@ -117,28 +114,38 @@ void choose_tiled(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may_
     fill_plan(m, n, k, best_variant, best_split, out);
 }
 
-// The streaming kernel with the K split that fills the CUs.
-void choose_streaming(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
+// Skinny shapes: the 64 x 256 tile with three LDS stages (two K blocks of b, 64 KB, in flight per workgroup) and
+// the K split that finishes soonest under a model in microseconds: a workgroup advances one K block in the time
+// the workgroups running together need to pull their 32 KB of b each from HBM at 5.5 TB/s, and never faster than
+// the 1.05 us a block's copies take to arrive; 2 us per round for the first block and the output; the partial
+// planes and the reduce launch as for the other tiles, with 4 us for the launch (the main kernel is short).
+// Measured with b streamed from HBM (inputs rotated through more than the 256 MB cache) against the 64 x 144
+// streaming kernel and the 64 x 128 tile: 64 x 18432 x 7168 34.3 us (split 3) against 37.7 and 38.4;
+// 64 x 7168 x 7168 20.4 against 32.4 and 21.0; 1 x 18432 x 7168 29.2 against 31.8 and 34.1;
+// 1 x 28672 x 4096 26.7 against 34.6 and 30.6.
+void choose_skinny(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may_split = true) {
     if (num_cus <= 0) num_cus = 256;
-    int kbt = k / KBLK;
-    // Bandwidth-bound family: stream B once with the 64x144 ring kernel.  Pick the K split that
-    // minimises (rounds over the CUs) x (K blocks per workgroup) x (bytes of B per workgroup and
-    // K block) plus the fp32 partial planes the split writes and reads back.
-    long tiles = cdiv(m, 64) * cdiv(n, 144);
-    double best = 0; int best_s = 1;
+    const int kbt = k / KBLK;
+    const long tiles = cdiv(m, 64) * cdiv(n, 256);
+    int best_s = 1; double best = 0;
     for (int s = 1; s <= 8 && s <= kbt; s++) {
-        double t_main = (double)cdiv(tiles * s, num_cus) * (double)cdiv(kbt, s) * 144.0 * 128.0;
-        double t_red = s > 1 ? 8.0 * s * (double)m * (double)n / num_cus : 0.0;
-        if (s == 1 || t_main + t_red < best) { best = t_main + t_red; best_s = s; }
+        if (s > 1 && !may_split) break;
+        const long wgs = tiles * s;
+        const double together = (double)(wgs < num_cus ? wgs : num_cus);
+        double t_block = together * 32768.0 / 5.5e6;
+        if (t_block < 1.05) t_block = 1.05;
+        double cost = (double)cdiv(wgs, num_cus) * (2.0 + (double)cdiv(kbt, s) * t_block);
+        if (s > 1) cost += 4.0 + 0.24 * s + 1.19e-6 * s * (double)m * (double)n;
+        if (s == 1 || cost < best) { best = cost; best_s = s; }
     }
-    fill_plan(m, n, k, FP8BS_VARIANT_SKINNY64x144, best_s, out);
+    fill_plan(m, n, k, FP8BS_VARIANT_T64x256S3, best_s, out);
 }
 
-// Shape-family rule.  A few rows against a very large B -> the streaming kernel (operands on 16-byte
-// boundaries, n a multiple of 8).  Everything else -> the tiled kernel.
-void choose(int m, int n, int k, int num_cus, bool aligned, fp8bs_plan_t* out) {
-    if (aligned && vector_shape(n) && streaming_shape(m, n, k)) choose_streaming(m, n, k, num_cus, out);
-    else choose_tiled(m, n, k, num_cus, out);
+// Shape-family rule.  A few rows against a large b -> the 64 x 256 three-stage tile.  Everything else -> the
+// tile and K split that the cost model of the tiled kernel picks.
+void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may_split = true) {
+    if (skinny_shape(m, n, k)) choose_skinny(m, n, k, num_cus, out, may_split);
+    else choose_tiled(m, n, k, num_cus, out, may_split);
 }
 
 // Order of the tiles of a grouped call (the row counts themselves are on the device).  With a tile or more of
@@ -212,7 +219,7 @@ const char* fp8bs_strerror(int status) {
 int fp8bs_plan(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     if (!out) return FP8BS_ERR_NULL_POINTER;
     if (m <= 0 || n <= 0 || k <= 0 || (k % KBLK) != 0) return FP8BS_ERR_BAD_SHAPE;
-    choose(m, n, k, num_cus, true, out);
+    choose(m, n, k, num_cus, out);
     return FP8BS_OK;
 }
 
@@ -242,10 +249,10 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
     }
     const bool simple = aligned && vector_shape(n);      // streaming kernels possible
     if (variant == FP8BS_VARIANT_AUTO) {
-        choose(m, n, k, fp8bs::device_cus(), aligned, &plan);
+        choose(m, n, k, fp8bs::device_cus(), &plan);
         if (split_k > 0) fill_plan(m, n, k, plan.variant, split_k, &plan);
         // the planned K split needs a workspace the caller did not bring: the best plan that needs none
-        else if (plan.split_k > 1 && (!ws || ws_bytes < plan.workspace_bytes)) choose_tiled(m, n, k, fp8bs::device_cus(), &plan, false);
+        else if (plan.split_k > 1 && (!ws || ws_bytes < plan.workspace_bytes)) choose(m, n, k, fp8bs::device_cus(), &plan, false);
     } else {
         VariantInfo vi{};
         if (!variant_info(variant, &vi)) return FP8BS_ERR_BAD_VARIANT;
@@ -284,7 +291,7 @@ int fp8bs_gemm_noalloc(const void* a, const void* b, const float* a_scale, const
     // the plan fp8bs_gemm would follow; its partial planes must fit the built-in array
     fp8bs_plan_t plan{};
     if (k > 0) {
-        choose(m, n, k, fp8bs::device_cus(), vector_aligned(a, b, c), &plan);
+        choose(m, n, k, fp8bs::device_cus(), &plan);
         if (plan.split_k > 1 && plan.workspace_bytes > (uint64_t)FP8BS_NOALLOC_SCRATCH_BYTES) return FP8BS_ERR_SCRATCH_LIMIT;
     }
     void* ws = nullptr;
@@ -311,12 +318,15 @@ int fp8bs_gemm_grouped_ex(const void* a, const void* b, const float* a_scale, co
     g.split_k = 1; g.kb_per_split = k / KBLK; g.band_h = 4; g.num_experts = num_experts;
     g.by_expert = group_order(total_rows, num_experts);
     if (variant == FP8BS_VARIANT_AUTO) {
-        // The 256x256 tile for every routing: measured with 32 experts of 8 .. 1024 rows each (even and
-        // random counts, n x k = 4096 x 7168 and 7168 x 2048) it is the fastest of the tiles throughout -
-        // with few rows per expert the call streams every expert's weights once and the waves without
-        // rows only copy, and the widest tile moves the fewest bytes of a per byte of b.  Any n and any
+        // The 256x256 tile for every routing with more than 32 rows per expert on average: measured with 32
+        // experts of 8 .. 1024 rows each (even and random counts, n x k = 4096 x 7168 and 7168 x 2048) it is the
+        // fastest of the two-stage tiles throughout - the waves without rows only copy, and the widest tile moves
+        // the fewest bytes of a per byte of b.  With 32 rows or fewer per expert the call streams every expert's
+        // weights once and little else: the 64 x 256 tile with three stages keeps two K blocks of b in flight per
+        // workgroup (32 experts x 4096 x 7168: 1 / 8 / 32 rows each 165 / 167 / 173 us against 181 / 185 / 186;
+        // from 100 rows on an expert needs a second row of its tiles and the 256x256 tile wins).  Any n and any
         // operand alignment (the instantiation that repairs every expert's last bytes of b).
-        variant = k != 0 ? FP8BS_VARIANT_T256x256 : FP8BS_VARIANT_GENERIC;
+        variant = k == 0 ? FP8BS_VARIANT_GENERIC : ((long)total_rows <= 32L * num_experts ? FP8BS_VARIANT_T64x256S3 : FP8BS_VARIANT_T256x256);
     } else {
         VariantInfo vi{};
         if (!variant_info(variant, &vi) || is_streaming_variant(variant)) return FP8BS_ERR_BAD_VARIANT;   // no grouped mode in the streaming kernels

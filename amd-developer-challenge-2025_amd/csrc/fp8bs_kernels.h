@@ -65,6 +65,7 @@ hipError_t launch_tile_256x128s3(const GemmArgs& args, int mode, hipStream_t str
 hipError_t launch_tile_128x128(const GemmArgs& args, int mode, hipStream_t stream);
 hipError_t launch_tile_64x128(const GemmArgs& args, int mode, hipStream_t stream);
 hipError_t launch_tile_192x192s3(const GemmArgs& args, int mode, hipStream_t stream);
+hipError_t launch_tile_64x256s3(const GemmArgs& args, int mode, hipStream_t stream);
 hipError_t launch_splitk_reduce(const float* ws, uint16_t* c, size_t mn, int split_k, hipStream_t stream);
 int variant_lds_bytes(int variant);
 

@@ -383,6 +383,7 @@ hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t str
         case 9: return launch_tile_256x192(a, mode, stream);
         case 10: return launch_tile_256x128s3(a, mode, stream);
         case 11: return launch_tile_192x192s3(a, mode, stream);
+        case 12: return launch_tile_64x256s3(a, mode, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -409,6 +410,7 @@ int variant_lds_bytes(int variant) {
         case 9: return TileCfg<256, 192, 64, 96, 0>::LDS_BYTES;
         case 10: return TileCfg<256, 128, 64, 64, 0, 3>::LDS_BYTES;
         case 11: return TileCfg<192, 192, 48, 96, 0, 3>::LDS_BYTES;
+        case 12: return TileCfg<64, 256, 32, 64, 0, 3>::LDS_BYTES;
         default: return 0;
     }
 }

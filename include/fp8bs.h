@@ -51,13 +51,15 @@ enum {
     FP8BS_VARIANT_T128x128 = 3,   /* mid-size: 128x128 tile, 4 waves                         */
     FP8BS_VARIANT_T64x128 = 4,    /* skinny-M: 64(m) x 128(n) tile, 4 waves, split-K         */
     FP8BS_VARIANT_T256x128 = 5,   /* 256(m) x 128(n) tile, 8 waves                           */
-    FP8BS_VARIANT_SKINNY64x144 = 6, /* bandwidth-bound: 64(m) x 144(n) tile, 4-stage copy ring */
+    FP8BS_VARIANT_SKINNY64x144 = 6, /* streaming kernel: 64(m) x 144(n) tile, 4-stage copy ring (forced only: needs m <= 64
+                                       per tile row to pay, n % 8 == 0 and operands on 16-byte boundaries) */
     FP8BS_VARIANT_SKINNY64x256 = 7, /* same, 256-wide tile (whole 128-byte lines), 3 stages      */
     FP8BS_VARIANT_SKINNY64x288 = 8, /* same, 288-wide tile, 3 stages                             */
     FP8BS_VARIANT_T256x192 = 9,   /* 256(m) x 192(n) tile, 8 waves: fills more CUs when n/256 rounds up badly */
     FP8BS_VARIANT_T256x128S3 = 10, /* 256 x 128 tile, three LDS stages (a copy has two K blocks' time to land) */
     FP8BS_VARIANT_T192x192S3 = 11, /* 192 x 192 tile, 8 waves of 48 x 96, three LDS stages     */
-    FP8BS_VARIANT_COUNT = 12
+    FP8BS_VARIANT_T64x256S3 = 12,  /* 64(m) x 256(n) tile, 8 waves of 32 x 64, three LDS stages: few rows against much of b */
+    FP8BS_VARIANT_COUNT = 13
 };
 
 /* What fp8bs_plan() decides for a shape. Replaces the exact-(m,n,k) if-ladder of the reference
@@ -81,10 +83,8 @@ const char* fp8bs_strerror(int status);
 
 /* Host-only planning: no GPU needed. Replaces the dispatch of
  * 1-amd-fp8-mm/amd-fp8-mm-submission.py:528-578. `num_cus` <= 0 means 256 (MI355X).  The plan is the one
- * fp8bs_gemm follows for operands on 16-byte boundaries and a workspace of workspace_bytes.  Operands off
- * that grid get the tiled plan for the shape where this one names the streaming kernel; without the
- * workspace of a planned K split fp8bs_gemm runs the best tiled plan that needs none (slower, same result
- * up to the summation order). */
+ * fp8bs_gemm follows with a workspace of workspace_bytes; without the workspace of a planned K split
+ * fp8bs_gemm runs the best plan that needs none (slower, same result up to the summation order). */
 int fp8bs_plan(int m, int n, int k, int num_cus, fp8bs_plan_t* out);
 
 /* Bytes of device workspace fp8bs_gemm needs for this shape (0 when split_k == 1). Replaces the
@@ -98,10 +98,8 @@ size_t fp8bs_workspace_bytes(int m, int n, int k);
  * Any m and n, a and b on any byte, c on any bf16 element: the tiled kernels read a and b with their
  * true row lengths, repair their last one to three bytes in LDS and, with n not a multiple of 8 or c off
  * the 16-byte grid, store c (and the partial planes of a K split) without assuming any alignment of its
- * rows; a workspace off the 16-byte grid is used from its first 16-byte boundary on; the streaming
- * kernel, planned for at most 64 rows against a very large b with n a multiple of 8 and operands on
- * 16-byte boundaries, repairs a the same way.  a_scale and b_scale must be 4-byte aligned, c 2-byte
- * aligned (FP8BS_ERR_BAD_SHAPE otherwise). */
+ * rows; a workspace off the 16-byte grid is used from its first 16-byte boundary on.  a_scale and b_scale
+ * must be 4-byte aligned, c 2-byte aligned (FP8BS_ERR_BAD_SHAPE otherwise). */
 int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
                void* c, void* ws, size_t ws_bytes, int m, int n, int k, void* stream);
 

@@ -30,8 +30,9 @@ def test_plan_shape_families(pkg):
     p = pkg.plan(4096, 4096, 4096)
     assert p.variant == 2 and (p.tile_m, p.tile_n) == (256, 256) and p.split_k == 1 and p.workspace_bytes == 0
     assert p.grid_x == 256 and p.block_threads == 512 and p.lds_bytes == 2 * (128 * 512 + 1024 + 256)     # A + B + a_scale row + b_scale values, two stages
-    p = pkg.plan(64, 18432, 7168)                       # skinny-M: streaming tile, split-K fills the CUs
-    assert p.variant == 6 and (p.tile_m, p.tile_n) == (64, 144) and p.split_k == 2 and p.grid_x == 256
+    p = pkg.plan(64, 18432, 7168)                       # skinny-M: the 64x256 tile with three stages, 72 tiles x a K split of 3
+    assert p.variant == 12 and (p.tile_m, p.tile_n) == (64, 256) and p.split_k == 3 and p.grid_x == 216
+    assert p.block_threads == 512 and p.lds_bytes == 3 * (128 * 320 + 1024 + 256)
     assert p.workspace_bytes == p.split_k * 64 * 18432 * 4 == pkg.workspace_bytes(64, 18432, 7168)
     p = pkg.plan(130, 190, 256)                         # n not a multiple of 8, short K -> a tiled kernel without a K split
     assert p.variant in (2, 3, 4, 9, 10, 11) and p.split_k == 1
@@ -40,10 +41,10 @@ def test_plan_shape_families(pkg):
     assert p.workspace_bytes == p.split_k * 1024 * 190 * 4
     for m in (130, 4095, 3, 1):                               # any m: the tiled kernels, one launch, nothing extra in the workspace
         p, q = pkg.plan(m, 192, 256), pkg.plan((m + 3) & ~3, 192, 256)
-        assert p.variant == q.variant and p.variant not in (1, 6, 7, 8) and p.split_k == q.split_k
+        assert p.variant == q.variant and p.variant not in (1, 6, 7, 8, 12) and p.split_k == q.split_k
         assert p.workspace_bytes == (p.split_k * m * 192 * 4 if p.split_k > 1 else 0)
-    p, q = pkg.plan(3, 18432, 7168), pkg.plan(4, 18432, 7168) # a few rows against a large b: the streaming kernel, any m
-    assert p.variant == q.variant == 6 and p.split_k == q.split_k and p.workspace_bytes == p.split_k * 3 * 18432 * 4
+    p, q = pkg.plan(3, 18432, 7168), pkg.plan(4, 18432, 7168) # a few rows against a large b: the same skinny plan for any m
+    assert p.variant == q.variant == 12 and p.split_k == q.split_k and p.workspace_bytes == p.split_k * 3 * 18432 * 4
     assert pkg.plan(3, 190, 256).variant in (3, 4)
     p = pkg.plan(256, 512, 1024)                        # small: one of the sub-256 tiles, never the scalar kernel
     assert p.variant in (3, 4, 10) and p.split_k >= 1 and p.split_k <= 8
@@ -59,19 +60,23 @@ def test_plan_shape_families(pkg):
     assert p.variant == 10 and (p.tile_m, p.tile_n) == (256, 128) and p.lds_bytes == 3 * (128 * 384 + 1024 + 256)
 
 
-def test_plan_streaming_kernel_only_for_few_rows_against_a_large_b(pkg):
-    """The streaming kernel is planned for at most 64 rows and a B of 96 MB or more; everything else goes
-    through the tiled kernels' cost model (more rows would make the streaming kernel copy B twice)."""
-    for m, n, k, streaming in [(64, 18432, 7168, True), (16, 18432, 7168, True), (4, 18432, 7168, True),
-                               (65, 18432, 7168, False), (128, 18432, 7168, False), (64, 7168, 7168, False),
-                               (64, 18432, 2048, False), (32, 512, 2048, False)]:
+def test_plan_skinny_tile_only_for_few_rows_against_a_large_b(pkg):
+    """The 64x256 three-stage tile is planned for at most 64 rows and a B of 24 MB or more; everything else goes
+    through the cost model of the other tiles (more rows would make it copy B twice).  The streaming kernels are
+    never planned (forced variants only)."""
+    for m, n, k, skinny in [(64, 18432, 7168, True), (16, 18432, 7168, True), (4, 18432, 7168, True), (64, 7168, 7168, True),
+                            (1, 28672, 4096, True), (64, 18440, 7168, True), (63, 18429, 7168, True),
+                            (65, 18432, 7168, False), (128, 18432, 7168, False), (64, 2048, 7168, False),
+                            (64, 7168, 2048, False), (32, 512, 2048, False)]:
         p = pkg.plan(m, n, k)
-        assert (p.variant in (6, 7, 8)) == streaming, (m, n, k, p.variant)
-        assert p.variant != 1
-        assert p.workspace_bytes == (p.split_k * m * n * 4 if p.split_k > 1 else 0)
+        assert (p.variant == 12) == skinny, (m, n, k, p.variant)
+        assert p.variant not in (1, 6, 7, 8)
+        assert 1 <= p.split_k <= 8 and p.workspace_bytes == (p.split_k * m * n * 4 if p.split_k > 1 else 0)
+        if skinny:
+            assert p.grid_x == -(-n // 256) * p.split_k
     for m in (1, 5, 63):                                      # rows that are not a multiple of four: the same plan
         p, q = pkg.plan(m, 18432, 7168), pkg.plan((m + 3) & ~3, 18432, 7168)
-        assert p.variant == q.variant == 6 and p.split_k == q.split_k
+        assert p.variant == q.variant == 12 and p.split_k == q.split_k
 
 
 def test_plan_rejects_bad_shapes(pkg):

@@ -11,7 +11,7 @@ from conftest import GOLDEN
 
 pytestmark = pytest.mark.gpu
 RTOL, ATOL = 2e-2, 1e-3
-MFMA_VARIANTS = (2, 3, 4, 5, 6, 7, 8, 9, 10, 11)
+MFMA_VARIANTS = (2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12)
 
 
 @pytest.fixture(scope="module")

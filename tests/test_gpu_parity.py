@@ -61,14 +61,14 @@ def test_config1_and_entry_point_contract(pkg, oracle, dev):
 
 def test_golden_fixture_bit_exact(pkg, golden_gemm, dev):
     cpu, expected, _ = golden_gemm
-    for variant in (0, 1, 3, 4, 6, 7, 8, 9, 10, 11): # planner's choice, generic, 128x128 tile, 64x128 tile, the three ring kernels, 256x192 tile, three-stage 256x128
+    for variant in (0, 1, 3, 4, 6, 7, 8, 9, 10, 11, 12): # planner's choice, generic, 128x128 tile, 64x128 tile, the three ring kernels, 256x192 tile, the three-stage tiles
         out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1 if variant else 0)
         assert torch.equal(out.cpu().view(torch.int16), expected.view(torch.int16)), "variant %d" % variant
     out = pkg.custom_kernel(_to(cpu, dev), variant=4, split_k=2)            # exact data: split-K is exact too
     assert torch.equal(out.cpu().view(torch.int16), expected.view(torch.int16))
 
 
-@pytest.mark.parametrize("variant,split_k", [(1, 1), (2, 1), (3, 1), (4, 1), (5, 1), (6, 1), (2, 2), (3, 3), (4, 4), (5, 8), (4, 7), (6, 2), (6, 8), (7, 1), (7, 2), (7, 3), (8, 1), (8, 4), (9, 1), (9, 2), (9, 8), (10, 1), (10, 2), (10, 3), (10, 4), (10, 8), (11, 1), (11, 2), (11, 3), (11, 8)])
+@pytest.mark.parametrize("variant,split_k", [(1, 1), (2, 1), (3, 1), (4, 1), (5, 1), (6, 1), (2, 2), (3, 3), (4, 4), (5, 8), (4, 7), (6, 2), (6, 8), (7, 1), (7, 2), (7, 3), (8, 1), (8, 4), (9, 1), (9, 2), (9, 8), (10, 1), (10, 2), (10, 3), (10, 4), (10, 8), (11, 1), (11, 2), (11, 3), (11, 8), (12, 1), (12, 2), (12, 3), (12, 7)])
 def test_every_variant_and_split_on_config1(pkg, oracle, dev, variant, split_k):
     cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0])
     out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=split_k)
@@ -96,13 +96,13 @@ def test_ragged_and_tail_shapes(pkg, oracle, dev, m, n, k):
     assert pkg.plan(m, n, k).variant != 1                       # any m and n: the vector kernels
     # every tile takes any m and n (the last bytes of a and b are repaired in LDS, a row's last chunk of
     # c is stored in pieces); the streaming kernels n % 8 == 0, and all but the planner's width m % 4 == 0
-    for variant in (2, 3, 4, 5, 9, 10, 11) + ((6,) if n % 8 == 0 else ()) + ((7, 8) if m % 4 == 0 and n % 8 == 0 else ()):
+    for variant in (2, 3, 4, 5, 9, 10, 11, 12) + ((6,) if n % 8 == 0 else ()) + ((7, 8) if m % 4 == 0 and n % 8 == 0 else ()):
         out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=1)
         _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d" % (m, n, k, variant))
     if k >= 256:
         # a K split on any n (partial planes written element by element where rows end inside a group of four,
         # reduction over the flat m*n array); the repair of a and b happens in the last split only
-        for variant in (4, 2, 11) + ((6,) if n % 8 == 0 else ()):
+        for variant in (4, 2, 11, 12) + ((6,) if n % 8 == 0 else ()):
             out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=2)
             _check(oracle, out, oracle.ref_kernel(cpu), "shape %dx%dx%d variant %d split 2" % (m, n, k, variant))
 
@@ -225,7 +225,7 @@ def test_pointers_off_the_16_byte_grid(pkg, oracle, dev, which, shift, m, n, k):
     _check(oracle, out, ref, "misaligned %s by %d" % (which, shift))
     if "c" in which:
         assert bool((buf[:off] == -7.0).all()) and bool((buf[off + m * n:] == -7.0).all()), "bytes outside c were written"
-    for variant in (2, 4, 9, 10, 11):
+    for variant in (2, 4, 9, 10, 11, 12):
         out = pkg.custom_kernel((a, b, a_scale, b_scale, c), variant=variant, split_k=1)
         _check(oracle, out, ref, "misaligned %s by %d, variant %d" % (which, shift, variant))
     with pytest.raises(RuntimeError):
@@ -257,7 +257,7 @@ def test_rows_not_a_multiple_of_four_without_a_workspace(pkg, oracle, dev, m, n,
     _check(oracle, with_ws, oracle.ref_kernel(cpu), "workspace %dx%dx%d" % (m, n, k))
 
 
-@pytest.mark.parametrize("m,n,k,variant", [(130, 190, 256, 0), (64, 1001, 128, 2), (33, 257, 128, 4), (260, 2111, 256, 9), (129, 127, 384, 10), (5, 3, 128, 3), (200, 391, 512, 11)])
+@pytest.mark.parametrize("m,n,k,variant", [(130, 190, 256, 0), (64, 1001, 128, 2), (33, 257, 128, 4), (260, 2111, 256, 9), (129, 127, 384, 10), (5, 3, 128, 3), (200, 391, 512, 11), (70, 515, 384, 12)])
 def test_nothing_is_written_outside_c(pkg, oracle, dev, m, n, k, variant):
     """c sits in the middle of a larger buffer of a sentinel value: with rows that end inside a 16-byte chunk
     the kernels store the last chunk of a row in pieces, and neither the bytes in front of c nor those behind
@@ -296,12 +296,12 @@ def test_streaming_kernel_every_row_count_up_to_48(pkg, oracle, dev):
 
 @pytest.mark.parametrize("m", [1, 3, 5, 18, 63])
 def test_decode_rows_against_a_large_b(pkg, oracle, dev, m):
-    """A few token rows against configuration 4's weights (132 MB): the streaming kernel with a K split,
+    """A few token rows against configuration 4's weights (132 MB): the 64x256 three-stage tile with a K split,
     row counts off the 4-row grid included (one to three rows: k rows of a shorter than a dword)."""
     cfg = pkg.inputs.CONFIGS[3]
     cpu = pkg.inputs.make_dense(cfg, m=m)
     plan = pkg.plan(m, cfg.n, cfg.k)
-    assert plan.variant == 6 and plan.split_k > 1
+    assert plan.variant == 12 and plan.split_k > 1
     out = pkg.custom_kernel(_to(cpu, dev))
     _check(oracle, out, oracle.ref_kernel(cpu), "decode %d rows" % m)
 
@@ -401,7 +401,7 @@ def test_grouped_small(pkg, oracle, dev, tokens, n, k, experts, topk):
     _check(oracle, out, oracle.ref_grouped(cpu), "grouped %s" % ((tokens, n, k, experts, topk),))
 
 
-@pytest.mark.parametrize("variant", [0, 3, 11])
+@pytest.mark.parametrize("variant", [0, 3, 11, 12])
 @pytest.mark.parametrize("tokens,n,k,experts,topk", [(200, 256, 256, 70, 3), (500, 136, 128, 127, 2), (500, 136, 128, 128, 2),
                                                       (300, 256, 128, 200, 4), (2048, 512, 256, 3, 2), (6000, 256, 128, 2, 1),
                                                       (3000, 384, 128, 9, 1)])
@@ -455,7 +455,7 @@ def test_grouped_every_element_against_the_scalar_kernel(pkg, dev):
     assert torch.equal(out2, out)
 
 
-@pytest.mark.parametrize("variant", [0, 2, 3, 4, 5, 9, 10, 11])
+@pytest.mark.parametrize("variant", [0, 2, 3, 4, 5, 9, 10, 11, 12])
 @pytest.mark.parametrize("tokens,experts,topk,n,k,shift", [(96, 8, 2, 190, 384, 0), (300, 5, 3, 1001, 256, 0), (37, 8, 3, 257, 128, 0),
                                                            (341, 4, 1, 2047, 128, 0), (130, 6, 2, 262, 256, 0), (96, 8, 2, 448, 384, 3), (200, 3, 2, 263, 256, 5)])
 def test_grouped_with_columns_off_the_8_column_grid_and_pointers_off_the_16_byte_grid(pkg, oracle, dev, variant, tokens, experts, topk, n, k, shift):
@@ -486,7 +486,7 @@ def test_grouped_with_columns_off_the_8_column_grid_and_pointers_off_the_16_byte
         assert torch.equal(out.view(torch.int16), big.view(torch.int16)), "the library's choice is not the 256x256 tile"
 
 
-@pytest.mark.parametrize("variant", [2, 3, 4, 5, 9, 10, 11])
+@pytest.mark.parametrize("variant", [2, 3, 4, 5, 9, 10, 11, 12])
 @pytest.mark.parametrize("tokens,experts,topk,n,k", [(96, 8, 2, 448, 384), (1024, 32, 8, 2112, 256), (40, 16, 1, 256, 128), (37, 8, 3, 264, 384), (341, 4, 1, 512, 128)])
 def test_grouped_with_every_tile_against_the_scalar_kernel(pkg, dev, variant, tokens, experts, topk, n, k):
     """Every tile shape in grouped mode: experts of a few rows, empty experts (40 tokens over 16 experts), expert boundaries inside a
