@@ -426,11 +426,11 @@ void gemm_tr_kernel(const GemmArgs p) {
         int P = wave * 64 + lane;
         int krow = P / C::CPR_A, ch = stored_to_chunk<C::CPR_A>(P % C::CPR_A, swz_of_krow<C::CPR_A>(krow));
         int col = t.m0 + 16 * ch;
-        // Grouped: a chunk of rows that all belong to a later expert is not fetched at all.  Its lanes get an
-        // offset at the end of the buffer, for which the range check of the load returns zeros without a
-        // memory access: a tile that holds an expert's last few rows then moves a few chunks of a per k row
-        // instead of the tile's sixteen.
-        const bool skip = MODE == 2 && col >= t.row_hi && a_bytes < 0x80000000u;
+        // A chunk of rows that all lie beyond the matrix, or that all belong to a later expert, is not fetched at
+        // all.  Its lanes get an offset at the end of the buffer, for which the range check of the load returns
+        // zeros without a memory access: one token row against a 64-row tile then moves one chunk of a per k row
+        // instead of four, a tile that holds an expert's last few rows a few instead of sixteen.
+        const bool skip = col >= t.row_hi && a_bytes < 0x80000000u;
         col = col < p.lda ? col : t.m0;
         c.a_voff = skip ? a_bytes : (uint32_t)krow * (uint32_t)p.lda + (uint32_t)col;
 #pragma unroll
@@ -440,15 +440,16 @@ void gemm_tr_kernel(const GemmArgs p) {
                 const int Pq = q * C::NWAVES * 64 + P;
                 const int kr = Pq / C::CPR_A;
                 int cl = t.m0 + 16 * stored_to_chunk<C::CPR_A>(Pq % C::CPR_A, swz_of_krow<C::CPR_A>(kr));
-                const bool skipq = MODE == 2 && cl >= t.row_hi && a_bytes < 0x80000000u;
+                const bool skipq = cl >= t.row_hi && a_bytes < 0x80000000u;
                 cl = cl < p.lda ? cl : t.m0;
                 c.a_voffq[q] = skipq ? a_bytes : (uint32_t)kr * (uint32_t)p.lda + (uint32_t)cl;
             }
         }
         krow = P / C::CPR_B; ch = stored_to_chunk<C::CPR_B>(P % C::CPR_B, swz_of_krow<C::CPR_B>(krow));
         col = t.n0 + 16 * ch;
+        const bool skip_b = col >= p.n && b_bytes < 0x80000000u;      // columns beyond the matrix: not fetched either
         col = col < p.n ? col : t.n0;
-        c.b_voff = (uint32_t)krow * (uint32_t)p.n + (uint32_t)col;
+        c.b_voff = skip_b ? b_bytes : (uint32_t)krow * (uint32_t)p.n + (uint32_t)col;
 #pragma unroll
         for (int q = 0; q < C::B_LOADS; q++) {
             c.b_voffq[q] = 0;
@@ -456,8 +457,9 @@ void gemm_tr_kernel(const GemmArgs p) {
                 const int Pq = q * C::NWAVES * 64 + P;
                 const int kr = Pq / C::CPR_B;
                 int cl = t.n0 + 16 * stored_to_chunk<C::CPR_B>(Pq % C::CPR_B, swz_of_krow<C::CPR_B>(kr));
+                const bool skipq = cl >= p.n && b_bytes < 0x80000000u;
                 cl = cl < p.n ? cl : t.n0;
-                c.b_voffq[q] = (uint32_t)kr * (uint32_t)p.n + (uint32_t)cl;
+                c.b_voffq[q] = skipq ? b_bytes : (uint32_t)kr * (uint32_t)p.n + (uint32_t)cl;
             }
         }
         int r = sc_is_b ? t.n0 / 128 + lane : t.m0 + wave * 64 + lane;      // n block or row of a
