@@ -138,7 +138,8 @@ int fp8bs_gemm_grouped(const void* a, const void* b, const float* a_scale, const
 
 /* Same with the tile forced: one of the FP8BS_VARIANT_T* tiles or FP8BS_VARIANT_GENERIC (the streaming
  * variants have no grouped mode: FP8BS_ERR_BAD_VARIANT).  FP8BS_VARIANT_AUTO reproduces
- * fp8bs_gemm_grouped (the 256x256 tile for any n and any operand alignment; the scalar kernel only for k = 0). */
+ * fp8bs_gemm_grouped (the 256x256 tile, or the 64x256 three-stage tile when total_rows <= 32 * num_experts, for any n
+ * and any operand alignment; the scalar kernel only for k = 0). */
 int fp8bs_gemm_grouped_ex(const void* a, const void* b, const float* a_scale, const float* b_scale,
                           void* c, const int32_t* row_offsets, int num_experts, int total_rows,
                           int n, int k, int variant, void* stream);
