@@ -461,8 +461,9 @@ def test_grouped_every_element_against_the_scalar_kernel(pkg, dev):
 def test_grouped_with_columns_off_the_8_column_grid_and_pointers_off_the_16_byte_grid(pkg, oracle, dev, variant, tokens, experts, topk, n, k, shift):
     """The grouped walk on the vector kernels with any n and any operand alignment: every expert's matrix of b
     loses its own last bytes when n is not a multiple of four (repaired per tile), rows of c are stored in
-    pieces.  Every element against the oracle, and the library's choice must be the 256x256 tile's result bit
-    for bit (not the scalar kernel's).  A poisoned margin around c stays untouched."""
+    pieces.  Every element against the oracle, and the library's choice (the 256x256 tile, or the 64x256 one for
+    a few rows per expert) must be the 256x256 tile's result bit for bit: every MFMA tile adds the same numbers in
+    the same order, the scalar kernel does not.  A poisoned margin around c stays untouched."""
     cfg = pkg.inputs.CONFIGS[4]
     cpu = pkg.inputs.make_grouped(cfg, tokens=tokens, experts=experts, topk=topk, n=n, k=k)
     a, b, a_scale, b_scale, row_offsets, c = _to(cpu, dev)
@@ -483,7 +484,7 @@ def test_grouped_with_columns_off_the_8_column_grid_and_pointers_off_the_16_byte
     assert bool((buf[:off] == -7.0).all()) and bool((buf[off + rows * n:] == -7.0).all()), "bytes outside c were written"
     if variant == 0:
         big = pkg.grouped_kernel((a, b, a_scale, b_scale, row_offsets, torch.empty_like(out)), variant=2)
-        assert torch.equal(out.view(torch.int16), big.view(torch.int16)), "the library's choice is not the 256x256 tile"
+        assert torch.equal(out.view(torch.int16), big.view(torch.int16)), "the library's choice is not an MFMA tile"
 
 
 @pytest.mark.parametrize("variant", [2, 3, 4, 5, 9, 10, 11, 12])
