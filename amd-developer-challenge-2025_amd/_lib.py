@@ -18,7 +18,7 @@ EXPORTS = (
     "fp8bs_gemm_silu_mul", "fp8bs_moe_combine", "fp8bs_convert_fnuz_to_fn", "fp8bs_diag_mfma_mix",
 )
 
-VARIANT_NAMES = {0: "auto", 1: "generic", 2: "t256x256", 3: "t128x128", 4: "t64x128", 5: "t256x128", 6: "skinny64x144", 7: "skinny64x256", 8: "skinny64x288", 9: "t256x192", 10: "t256x128s3", 11: "t192x192s3"}
+VARIANT_NAMES = {0: "auto", 1: "generic", 2: "t256x256", 3: "t128x128", 4: "t64x128", 5: "t256x128", 6: "skinny64x144", 7: "skinny64x256", 8: "skinny64x288", 9: "t256x192", 10: "t256x128s3", 11: "t192x192s3", 12: "t64x256s3"}
 
 
 class Plan(ctypes.Structure):
@@ -27,7 +27,7 @@ class Plan(ctypes.Structure):
         ("variant", ctypes.c_int32), ("tile_m", ctypes.c_int32), ("tile_n", ctypes.c_int32),
         ("split_k", ctypes.c_int32), ("grid_x", ctypes.c_int32), ("grid_y", ctypes.c_int32),
         ("grid_z", ctypes.c_int32), ("block_threads", ctypes.c_int32), ("lds_bytes", ctypes.c_int32),
-        ("reserved", ctypes.c_int32), ("workspace_bytes", ctypes.c_uint64),
+        ("stream_k", ctypes.c_int32), ("workspace_bytes", ctypes.c_uint64),
     ]
 
 

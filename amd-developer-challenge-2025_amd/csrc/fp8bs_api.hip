@@ -8,6 +8,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stddef.h>
+#include <stdlib.h>
+#include <unistd.h>
+#include <atomic>
+#include <chrono>
 
 #include "fp8bs.h"
 #include "fp8bs_kernels.h"
@@ -38,12 +42,29 @@ bool variant_info(int variant, VariantInfo* out) {
 
 inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 
+// Workgroups of a call that deals K blocks instead of tiles: one per place on the chip (what the tile's LDS
+// and thread count let a CU hold), never more than there are (tile, K block) pairs.
+int streamk_grid(int variant, int m, int n, int k, int num_cus) {
+    VariantInfo vi{};
+    if (!variant_info(variant, &vi) || variant == FP8BS_VARIANT_GENERIC || k < KBLK) return 0;
+    const int lds = fp8bs::variant_lds_bytes(variant);
+    if (lds <= 0 || lds > 163840) return 0;
+    if (num_cus <= 0) num_cus = 256;
+    const long by_lds = 163840 / lds, by_threads = 2048 / vi.threads;
+    long g = (long)num_cus * (by_lds < by_threads ? by_lds : by_threads);
+    const long pairs = cdiv(m, vi.bm) * cdiv(n, vi.bn) * (k / KBLK);
+    if (pairs >= (1L << 31)) return 0;                  // the kernel counts the pairs in 32 bits
+    g = g < pairs ? g : pairs;
+    return (int)(g < fp8bs::StreamK::MAX_GRID ? g : fp8bs::StreamK::MAX_GRID);
+}
+
 // Fill a plan for a given variant and split count.
-void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out) {
+void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out, int stream_k = 0) {
     VariantInfo vi{};
     variant_info(variant, &vi);
     int kbt = k / KBLK;
-    if (variant == FP8BS_VARIANT_GENERIC) split_k = 1;
+    if (variant == FP8BS_VARIANT_GENERIC) { split_k = 1; stream_k = 0; }
+    if (stream_k > 0) split_k = 1;
     if (split_k < 1) split_k = 1;
     if (split_k > kbt) split_k = kbt > 0 ? kbt : 1;
     out->variant = variant;
@@ -52,13 +73,14 @@ void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out)
     out->split_k = split_k;
     out->block_threads = vi.threads;
     out->lds_bytes = fp8bs::variant_lds_bytes(variant);
-    out->reserved = 0;
+    out->stream_k = stream_k > 0 ? stream_k : 0;
     if (variant == FP8BS_VARIANT_GENERIC) {
         out->grid_x = (int)cdiv(n, 16); out->grid_y = (int)cdiv(m, 16); out->grid_z = 1;
     } else {
-        out->grid_x = (int)(cdiv(m, vi.bm) * cdiv(n, vi.bn) * split_k); out->grid_y = 1; out->grid_z = 1;
+        out->grid_x = stream_k > 0 ? stream_k : (int)(cdiv(m, vi.bm) * cdiv(n, vi.bn) * split_k); out->grid_y = 1; out->grid_z = 1;
     }
-    out->workspace_bytes = split_k > 1 ? (uint64_t)split_k * (uint64_t)m * (uint64_t)n * 4u : 0u;
+    out->workspace_bytes = stream_k > 0 ? (uint64_t)fp8bs::StreamK::bytes(stream_k, vi.bm, vi.bn)
+                                        : (split_k > 1 ? (uint64_t)split_k * (uint64_t)m * (uint64_t)n * 4u : 0u);
 }
 
 // Rows of c (n bf16) that keep 16-byte stores aligned: what the streaming kernels need (forced variants only;
@@ -155,6 +177,28 @@ void choose(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may_split 
 // the order across the experts is then 0.7-1.2 % ahead (8 or 100 rows per expert), so it is kept there.
 int group_order(int total_rows, int num_experts) { return (long)total_rows >= 256L * num_experts ? 1 : 0; }
 
+// The value a flag takes in one call that deals K blocks: never zero, different from call to call (and, through
+// the clock and the process id, from run to run), so that whatever an earlier call or an uninitialised workspace
+// left in a flag is not mistaken for this call's.
+unsigned long long next_nonce() {
+    static std::atomic<unsigned long long> counter{0};
+    static const unsigned long long seed = ((unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count() * 0x9E3779B97F4A7C15ull)
+                                           ^ ((unsigned long long)getpid() << 32);
+    unsigned long long x = seed + (counter.fetch_add(1, std::memory_order_relaxed) + 1) * 0xD1342543DE82EF95ull;
+    return x ? x : 1ull;
+}
+
+// Polls of one flag before a workgroup's wait gives up (each poll is a round trip to memory plus a short sleep,
+// about a microsecond: the default is a quarter of a second or so).  FP8BS_STREAMK_SPIN overrides it; a negative
+// value makes every such wait give up at once, which exercises the error path without a kernel that hangs.
+int streamk_spin_limit() {
+    static const int limit = [] {
+        const char* e = getenv("FP8BS_STREAMK_SPIN");
+        return e && *e ? atoi(e) : (1 << 18);
+    }();
+    return limit;
+}
+
 bool is_streaming_variant(int v) { return v == FP8BS_VARIANT_SKINNY64x144 || v == FP8BS_VARIANT_SKINNY64x256 || v == FP8BS_VARIANT_SKINNY64x288; }
 
 int check_common(const void* a, const void* b, const float* as, const float* bs, void* c, int m, int n, int k) {
@@ -211,6 +255,7 @@ const char* fp8bs_strerror(int status) {
         case FP8BS_ERR_LAUNCH: return "kernel launch failed";
         case FP8BS_ERR_BAD_OFFSETS: return "grouped: num_experts must be positive";
         case FP8BS_ERR_BAD_VARIANT: return "unknown or inapplicable kernel variant";
+        case FP8BS_ERR_TIMEOUT: return "a workgroup gave up waiting for another workgroup's partial tile (status word of the workspace); the output of that call is not valid";
         case FP8BS_ERR_SCRATCH_LIMIT: return "fp8bs_gemm_noalloc: the K split planned for this shape needs more than the built-in scratch (FP8BS_NOALLOC_SCRATCH_BYTES); use fp8bs_gemm with a caller workspace";
         default: return "unknown fp8bs status";
     }
@@ -248,19 +293,26 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
         else { ws = nullptr; ws_bytes = 0; }
     }
     const bool simple = aligned && vector_shape(n);      // streaming kernels possible
+    const int cus = fp8bs::device_cus();
     if (variant == FP8BS_VARIANT_AUTO) {
-        choose(m, n, k, fp8bs::device_cus(), &plan);
+        choose(m, n, k, cus, &plan);
         if (split_k > 0) fill_plan(m, n, k, plan.variant, split_k, &plan);
-        // the planned K split needs a workspace the caller did not bring: the best plan that needs none
-        else if (plan.split_k > 1 && (!ws || ws_bytes < plan.workspace_bytes)) choose(m, n, k, fp8bs::device_cus(), &plan, false);
+        else if (split_k < 0) fill_plan(m, n, k, plan.variant, 1, &plan, streamk_grid(plan.variant, m, n, k, cus));
+        // the plan needs a workspace the caller did not bring: the best plan that needs none
+        else if (plan.workspace_bytes > 0 && (!ws || ws_bytes < plan.workspace_bytes)) choose(m, n, k, cus, &plan, false);
     } else {
         VariantInfo vi{};
         if (!variant_info(variant, &vi)) return FP8BS_ERR_BAD_VARIANT;
         if (is_streaming_variant(variant) && !simple) return FP8BS_ERR_BAD_VARIANT;
         if (is_streaming_variant(variant) && variant != FP8BS_VARIANT_SKINNY64x144 && (m % 4) != 0) return FP8BS_ERR_BAD_VARIANT;   // only the planner's width repairs a
-        fill_plan(m, n, k, variant, split_k > 0 ? split_k : 1, &plan);
+        if (split_k < 0) {
+            if (is_streaming_variant(variant) || variant == FP8BS_VARIANT_GENERIC) return FP8BS_ERR_BAD_VARIANT;   // K blocks are dealt by the tiled kernel only
+            fill_plan(m, n, k, variant, 1, &plan, streamk_grid(variant, m, n, k, cus));
+        } else {
+            fill_plan(m, n, k, variant, split_k > 0 ? split_k : 1, &plan);
+        }
     }
-    if (plan.split_k > 1 && (!ws || ws_bytes < (uint64_t)plan.split_k * (uint64_t)m * (uint64_t)n * 4u)) return FP8BS_ERR_WORKSPACE;
+    if (plan.workspace_bytes > 0 && (!ws || ws_bytes < plan.workspace_bytes)) return FP8BS_ERR_WORKSPACE;
 
     fp8bs::GemmArgs g{};
     g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.as = a_scale; g.bs = b_scale;
@@ -271,6 +323,12 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
     g.band_h = 4;
     g.num_experts = 0;
     int mode = plan.split_k > 1 ? 1 : 0;
+    if (plan.stream_k > 0) {
+        mode = 3;
+        g.sk_grid = plan.stream_k;
+        g.sk_nonce = next_nonce();
+        g.sk_spin = streamk_spin_limit();
+    }
     if (fp8bs::launch_gemm(plan.variant, mode, g, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
     if (mode == 1) {
         if (fp8bs::launch_splitk_reduce(g.ws, g.c, (size_t)m * n, plan.split_k, s) != hipSuccess) return FP8BS_ERR_LAUNCH;
@@ -292,7 +350,7 @@ int fp8bs_gemm_noalloc(const void* a, const void* b, const float* a_scale, const
     fp8bs_plan_t plan{};
     if (k > 0) {
         choose(m, n, k, fp8bs::device_cus(), &plan);
-        if (plan.split_k > 1 && plan.workspace_bytes > (uint64_t)FP8BS_NOALLOC_SCRATCH_BYTES) return FP8BS_ERR_SCRATCH_LIMIT;
+        if (plan.workspace_bytes > (uint64_t)FP8BS_NOALLOC_SCRATCH_BYTES) return FP8BS_ERR_SCRATCH_LIMIT;
     }
     void* ws = nullptr;
     st = scratch_address(&ws);

@@ -25,6 +25,22 @@ struct GemmArgs {
     int epi;                // 0: bf16 of the product; 1: silu(column 2i) * column 2i+1, n/2 output columns
     int c_whole_lines;      // set by the launcher: rows of c start and end on 128-byte lines
     int by_expert;          // grouped: order of the tiles, 0 across the experts, 1 expert by expert (see the tile walk)
+    // K blocks dealt to the workgroups (MODE 3 of the tiled kernel): `ws` then holds a header (a status word, one
+    // 8-byte flag per workgroup) and one fp32 partial tile per workgroup, see StreamK below
+    unsigned long long sk_nonce;   // value a flag takes when its workgroup's partial tile is complete: differs from call to call
+    int sk_grid;            // workgroups of such a call: at most the places on the chip and the number of (tile, K block) pairs
+    int sk_spin;            // polls of a flag before the wait gives up (< 0: give up at once - tests of the error path)
+};
+
+// Workspace of a call that deals K blocks (all offsets from the 16-byte aligned workspace base):
+//   [0, 4)                          status word: set to FP8BS_ERR_TIMEOUT by a workgroup whose bounded wait gave up
+//   [SK_FLAGS_OFF, + 8 * grid)      one flag per workgroup
+//   [SK_SLOTS_OFF, + grid * slot)   one partial tile per workgroup, slot = tile_m * tile_n * 4 bytes, in lane order
+struct StreamK {
+    static constexpr size_t FLAGS_OFF = 256, SLOTS_OFF = 16384;
+    static constexpr int MAX_GRID = (int)((SLOTS_OFF - FLAGS_OFF) / 8);
+    static constexpr unsigned STATUS_TIMEOUT = 9;        // FP8BS_ERR_TIMEOUT
+    static size_t bytes(int grid, int tile_m, int tile_n) { return SLOTS_OFF + (size_t)grid * (size_t)tile_m * (size_t)tile_n * 4u; }
 };
 
 // Per-device bookkeeping of the launchers.  A kernel's dynamic-LDS limit is a property of the kernel

@@ -247,6 +247,7 @@ void gemm_tr_kernel(const GemmArgs p) {
     // epilogue are a third of a tile's time otherwise).
     struct Tile {
         int valid, m0, n0, kb_begin, kb_end, split_z, row_lo, row_hi;
+        int sk_contrib, sk_first;             // MODE 3: the segment ends before the tile's last K block; first workgroup of the tile's earlier segments (-1: none)
         const uint8_t* bptr;
         const float* bsptr;
     };
@@ -293,12 +294,52 @@ void gemm_tr_kernel(const GemmArgs p) {
             }
         }
     }
+    [[maybe_unused]] const int sk_self = xcd_virtual_id(blockIdx.x, gridDim.x);
     auto pick_tile = [&](int it) -> Tile {
         Tile t;
         t.valid = 0; t.m0 = 0; t.n0 = 0; t.kb_begin = 0; t.kb_end = 0; t.split_z = 0; t.row_lo = 0; t.row_hi = p.m;
+        t.sk_contrib = 0; t.sk_first = -1;
         t.bptr = p.b; t.bsptr = p.bs;
         const int G = gridDim.x;
-        if (MODE == 2) {
+        if (MODE == 3) {
+            // K blocks, not tiles, are dealt to the workgroups: the (tile, K block) pairs of the whole product
+            // form one sequence - tiles in the band order of the dense walk, K ascending inside a tile - and
+            // workgroup v takes the run of total/G pairs (the first total%G runs hold one more), G <= total.  A run covers the end of one tile,
+            // whole tiles, and the beginning of another; the workgroup walks its tiles from the last to the
+            // first.  A segment that ends before its tile's last K block is stored as an fp32 partial tile in
+            // the workgroup's slot of the workspace (only the first segment a workgroup works on can be one);
+            // the segment that holds the tile's last K block belongs to the tile's owner, who adds the
+            // partial tiles of the workgroups before it in ascending order of K, then its own accumulators,
+            // and writes the output.  The owner works on that segment last and every workgroup it waits for
+            // has a lower index, started no later and worked on its partial tile first.
+            const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
+            const uint32_t kbt = (uint32_t)(p.k / KBLK);
+            const uint32_t total = (uint32_t)tiles_m * (uint32_t)tiles_n * kbt;           // < 2^31 (checked by the launcher)
+            // runs of q or q+1 pairs, the longer ones first
+            const uint32_t q = total / (uint32_t)G, r = total - q * (uint32_t)G;
+            auto run_start = [&](uint32_t w) -> uint32_t { return w * q + (w < r ? w : r); };
+            const uint32_t v = (uint32_t)sk_self;
+            const uint32_t s = run_start(v), e = run_start(v + 1);
+            if (e <= s) return t;
+            const int t_first = (int)(s / kbt), t_last = (int)((e - 1) / kbt);
+            const int tile = t_last - it;
+            if (tile < t_first) return t;
+            t.valid = 1;
+            int tm, tn;
+            band_tile(tile, tiles_m, tiles_n, p.band_h, tm, tn);
+            const uint32_t x0 = (uint32_t)tile * kbt;                                      // the tile's first pair
+            int kb0 = tile == t_first ? (int)(s - x0) : 0;
+            int kb1 = tile == t_last ? (int)(e - x0) : (int)kbt;
+            int first = -1;
+            if (kb1 == (int)kbt && kb0 > 0)                                               // the workgroup whose run holds x0
+                first = (int)(x0 < r * (q + 1) ? x0 / (q + 1) : r + (x0 - r * (q + 1)) / q);
+            // (uniform values that went through the vector ALU's division sequences: back to scalar registers)
+            t.m0 = __builtin_amdgcn_readfirstlane(tm * BM); t.n0 = __builtin_amdgcn_readfirstlane(tn * BN);
+            t.kb_begin = __builtin_amdgcn_readfirstlane(kb0);
+            t.kb_end = __builtin_amdgcn_readfirstlane(kb1);
+            t.sk_contrib = t.kb_end < (int)kbt;
+            t.sk_first = __builtin_amdgcn_readfirstlane(first);
+        } else if (MODE == 2) {
             // grouped: m-tile slots are laid over the experts in order; expert e's tiles start at
             // row_offsets[e] rounded down to 16 so that global 16-byte loads stay aligned; rows outside
             // [row_offsets[e], row_offsets[e+1]) are computed but never stored.  The gridDim.x tiles in
@@ -588,6 +629,7 @@ void gemm_tr_kernel(const GemmArgs p) {
     for (int it = 0;; it++) {
     const int m0 = cur.m0, n0 = cur.n0, kb_begin = cur.kb_begin, kb_end = cur.kb_end, split_z = cur.split_z;
     const int row_lo = cur.row_lo, row_hi = cur.row_hi;
+    [[maybe_unused]] const int sk_contrib = cur.sk_contrib, sk_first = cur.sk_first;
     if constexpr (TAILS && MODE == 2) {
         if (b_tail) b_last = __builtin_amdgcn_readfirstlane(load_last_dword(cur.bptr + ((uint32_t)p.k * (uint32_t)p.n - 4u)));
     }
@@ -789,8 +831,87 @@ void gemm_tr_kernel(const GemmArgs p) {
         }
     }
 
+    // ---- K blocks dealt to the workgroups: partial tiles travel through the workspace ---------------
+    // Partial tiles are written and read with agent-scope accesses (sc1: written through to, and read from,
+    // the memory side of the eight L2s), in the order of the lanes: the two sides run the same tile shape, so
+    // accumulator (t, u) of wave w is the 1 KiB piece number w*MT*NT + t*NT + u of the slot.
+    bool store_output = true;
+    if constexpr (MODE == 3) {
+        constexpr uint32_t SLOT_BYTES = (uint32_t)BM * (uint32_t)BN * 4u;
+        constexpr int NG = C::MT * C::NT;
+        constexpr int AUX_AGENT = 16;                                           // sc1
+        unsigned char* const ws_base = (unsigned char*)p.ws;
+        unsigned long long* const flags = (unsigned long long*)(ws_base + StreamK::FLAGS_OFF);
+        unsigned char* const slots = ws_base + StreamK::SLOTS_OFF;
+        if (sk_contrib) {
+            store_output = false;
+            if (wave_active) {
+                // (the accumulators are next written after the wait below: nothing follows these stores closely)
+                __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(slots + (size_t)sk_self * SLOT_BYTES), 0, SLOT_BYTES, 0x00020000);
+                const uint32_t voff = (uint32_t)(wave * NG) * 1024u + (uint32_t)lane * 16u;
+#pragma unroll
+                for (int t = 0; t < C::MT; t++)
+#pragma unroll
+                    for (int u = 0; u < C::NT; u++)
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, acc[t][u]), rs, voff + (uint32_t)(t * C::NT + u) * 1024u, 0, AUX_AGENT);
+            }
+            // A store with sc1 is written through to the agent's point of coherence and is counted by vmcnt
+            // until it is acknowledged from there, so after this wait every wave's part of the tile can be
+            // seen by any CU that reads it with sc1; the barrier then lets one lane raise the flag for all.
+            // (An agent-scope release fence in its place writes the whole L2 back once per wave: 4096 x 2112
+            // x 7168 took 131 us with it against 81 us, 64 x 18432 x 7168 76 us against 30 us.)
+            wait_vmcnt<0>();
+            __syncthreads();
+            if (tid == 0) __hip_atomic_store(&flags[sk_self], p.sk_nonce, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else if (sk_first >= 0) {
+            // The tile's owner: wait, a bounded number of polls, for the flags of the workgroups that hold the
+            // tile's earlier K blocks (one lane per flag, all polled together), take the flags down again (so
+            // that a replay of the same launch starts clean), then add the partial tiles to the accumulators in
+            // ascending order of K: ((own + P_first) + P_next) + ...  A wait that gives up leaves the status
+            // word set and the kernel runs on to its end with whatever the slots hold.
+            if (wave == 0) {
+                bool ok = p.sk_spin >= 0;
+                for (int base = sk_first; ok && base < sk_self; base += 64) {
+                    const int u = base + lane;
+                    const bool mine = u < sk_self;
+                    int spins = p.sk_spin;
+                    for (;;) {
+                        const unsigned long long f = mine ? __hip_atomic_load(&flags[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : p.sk_nonce;
+                        if (__ballot(f != p.sk_nonce) == 0) break;
+                        if (--spins < 0) { ok = false; break; }
+                        __builtin_amdgcn_s_sleep(2);
+                    }
+                    if (ok && mine) __hip_atomic_store(&flags[u], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                if (!ok && lane == 0) __hip_atomic_store((unsigned int*)ws_base, StreamK::STATUS_TIMEOUT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            __syncthreads();
+            if (wave_active) {
+                // loads in flight at a time: what the registers beside the accumulators hold
+                constexpr int BATCH = NG <= 8 ? NG : (NG % 4 == 0 ? 4 : (NG % 3 == 0 ? 3 : 1));
+                __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)slots, 0, (uint32_t)gridDim.x * SLOT_BYTES, 0x00020000);
+                const uint32_t voff = (uint32_t)(wave * NG) * 1024u + (uint32_t)lane * 16u;
+#pragma unroll
+                for (int base = 0; base < NG; base += BATCH) {
+#pragma unroll 2
+                    for (int u = sk_first; u < sk_self; u++) {
+                        const uint32_t soff = (uint32_t)u * SLOT_BYTES + (uint32_t)base * 1024u;
+                        v4f part[BATCH];
+#pragma unroll
+                        for (int i = 0; i < BATCH; i++)
+                            part[i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff + i * 1024u, AUX_AGENT));
+#pragma unroll
+                        for (int i = 0; i < BATCH; i++)
+                            acc[(base + i) / C::NT][(base + i) % C::NT] += part[i];
+                    }
+                    __builtin_amdgcn_sched_barrier(0);      // the registers hold the whole tile already: one batch at a time
+                }
+            }
+        }
+    }
+
     // ---- epilogue (a wave without valid rows has nothing to store; no barrier in here) -----------
-    if (!wave_active) {
+    if (!wave_active || !store_output) {
     } else if (MODE == 1) {
         // split-K: fp32 partial tile, 16 bytes per lane
 #pragma unroll
@@ -913,7 +1034,7 @@ void gemm_tr_kernel(const GemmArgs p) {
         }
     }
     if (!nxt.valid) break;
-    stores_behind = prefetched && wave_active && MODE != 1 && !TAILS;   // (with TAILS the store count is four times EPI_STORES: plain wait)
+    stores_behind = prefetched && wave_active && MODE != 1 && !TAILS && store_output;   // (with TAILS the store count is four times EPI_STORES: plain wait)
     cur = nxt; cp = ncp;
     }   // tiles
 }
@@ -957,6 +1078,14 @@ static inline hipError_t launch_shape(const GemmArgs& a, int mode, hipStream_t s
         total = (((long)a.m + BM - 1) / BM + 2L * a.num_experts) * tiles_n;
     } else {
         total = (long)((a.m + BM - 1) / BM) * tiles_n * a.split_k;
+    }
+    if (mode == 3) {
+        // K blocks dealt to the workgroups: one workgroup per place on the chip, never more than there are
+        // (tile, K block) pairs, so that every workgroup's run holds at least one
+        if (a.epi != 0 || a.k < KBLK) return hipErrorInvalidValue;
+        const long pairs = (long)((a.m + BM - 1) / BM) * tiles_n * (a.k / KBLK);
+        if (a.sk_grid < 1 || a.sk_grid > resident || a.sk_grid > pairs || a.sk_grid > StreamK::MAX_GRID) return hipErrorInvalidValue;
+        return launch_tr<BM, BN, WM, WN, 3, 0, NSTAGE>(a, dim3((unsigned)a.sk_grid), stream);
     }
     const dim3 grid((unsigned)(total < resident ? total : resident));
     if (a.epi != 0) {

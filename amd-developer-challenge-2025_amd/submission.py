@@ -173,7 +173,9 @@ def custom_kernel(data, variant: int = 0, split_k: int = 0):
             _plan_cache[(m, n, k)] = need
         _remember(key, data, m, n, k, need, a.device.index)
     else:
-        need = max(split_k, 1) * m * n * 4 if split_k > 1 else 0
+        # a forced K split's planes; K blocks dealt to the workgroups (split_k < 0): a header and one fp32 tile per
+        # workgroup, at most 64 MiB for every tile shape on 256 CUs
+        need = split_k * m * n * 4 if split_k > 1 else ((64 << 20) + 16384 if split_k < 0 else 0)
     # kernels are launched on the device the pointers live on: the library uses the current device
     with torch.cuda.device(a.device):
         stream = _stream_ptr(a.device)

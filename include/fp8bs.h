@@ -39,8 +39,11 @@ enum {
     FP8BS_ERR_LAUNCH = 5,         /* hipGetLastError() after launch was not hipSuccess       */
     FP8BS_ERR_BAD_OFFSETS = 6,    /* grouped: bad expert count                               */
     FP8BS_ERR_BAD_VARIANT = 7,    /* forced variant id unknown or not applicable             */
-    FP8BS_ERR_SCRATCH_LIMIT = 8   /* fp8bs_gemm_noalloc: the shape's K split needs more than
+    FP8BS_ERR_SCRATCH_LIMIT = 8,  /* fp8bs_gemm_noalloc: the shape's K split needs more than
                                      FP8BS_NOALLOC_SCRATCH_BYTES of partial planes            */
+    FP8BS_ERR_TIMEOUT = 9         /* never returned by a call (calls do not wait for the GPU): the value a
+                                     kernel leaves in the first word of the workspace when a workgroup's
+                                     bounded wait for another workgroup's partial tile gave up     */
 };
 
 /* Kernel variants the planner chooses from. */
@@ -71,7 +74,8 @@ typedef struct fp8bs_plan_t {
     int32_t grid_x, grid_y, grid_z;
     int32_t block_threads;
     int32_t lds_bytes;
-    int32_t reserved;
+    int32_t stream_k;       /* > 0: K blocks, not tiles, are dealt to this many workgroups (one launch;
+                               partial tiles meet in the workspace); split_k is 1 then           */
     uint64_t workspace_bytes;
 } fp8bs_plan_t;
 

@@ -10,9 +10,29 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "libfp8bs_oracle.so")
 
 
+PROBE_LIB = os.path.join(HERE, "libmfma_probe.so")
+
+
 def build() -> str:
-    subprocess.run(["make", "-s", "-B", "-C", HERE], check=True)
+    """Both checker libraries: the C restatement (host compiler) and the MFMA probe (hipcc, gfx950)."""
+    subprocess.run(["make", "-s", "-B", "-C", HERE, "all"], check=True, stdout=subprocess.DEVNULL if os.environ.get("ORACLE_QUIET") else None)
     return LIB
+
+
+_probe = None
+
+
+def load_probe() -> ctypes.CDLL:
+    """oracle/libmfma_probe.so (built ahead of time by build(); GPU runs load what is there)."""
+    global _probe
+    if _probe is None:
+        if not os.path.exists(PROBE_LIB):
+            raise RuntimeError("oracle/libmfma_probe.so is not built: run `make -C oracle` (needs hipcc)")
+        lib = ctypes.CDLL(PROBE_LIB)
+        lib.mfma_probe_chain_16x16x32.restype = ctypes.c_int
+        lib.mfma_probe_chain_16x16x32.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        _probe = lib
+    return _probe
 
 
 _lib = None
@@ -22,7 +42,7 @@ def load() -> ctypes.CDLL:
     global _lib
     if _lib is None:
         if not os.path.exists(LIB):
-            build()
+            subprocess.run(["make", "-s", "-C", HERE, "libfp8bs_oracle.so"], check=True)
         lib = ctypes.CDLL(LIB)
         lib.fp8bs_ref_e4m3fn_to_float.restype = ctypes.c_float
         lib.fp8bs_ref_e4m3fn_to_float.argtypes = [ctypes.c_uint8]

@@ -203,6 +203,46 @@ void fp8bs_model_gemm_at(const uint8_t* a, const uint8_t* b, const float* as, co
     }
 }
 
+/* Selected elements of a call that deals K blocks, not tiles, to the workgroups (fp8bs_gemm_ex with split_k < 0):
+ * the K blocks of the tile_m x tile_n tile T = (i / tile_m) * tiles_n + j / tile_n are cut at
+ * seg_bounds[seg_off[T]] = 0 < ... < seg_bounds[seg_off[T + 1] - 1] = K / 128; every piece is accumulated from
+ * zero in ascending K; the tile's owner holds the last piece and adds the others to it in ascending order:
+ * ((own + P_0) + P_1) + ...; one rounding to bf16. */
+void fp8bs_model_gemm_at_segments(const uint8_t* a, const uint8_t* b, const float* as, const float* bs, int m, int n, int k,
+                                  int tile_m, int tile_n, const int32_t* seg_off, const int32_t* seg_bounds,
+                                  const int32_t* idx, int count, uint16_t* out, float* out_f32) {
+    init_tables();
+    const int nb = (n + 127) / 128, lda = m, tiles_n = (n + tile_n - 1) / tile_n;
+    (void)k;
+#pragma omp parallel for schedule(dynamic, 16)
+    for (int t = 0; t < count; t++) {
+        const int i = idx[2 * t], j = idx[2 * t + 1];
+        const int T = (i / tile_m) * tiles_n + j / tile_n;
+        const int32_t* bd = seg_bounds + seg_off[T];
+        const int pieces = seg_off[T + 1] - seg_off[T] - 1;
+        uint8_t av[128], bv[128];
+        float part[64];
+        float own = 0.0f;
+        for (int z = 0; z < pieces; z++) {
+            float acc = 0.0f;
+            for (int kb = bd[z]; kb < bd[z + 1]; kb++) {
+                for (int r = 0; r < 128; r++) {
+                    const int x = 32 * ((r >> 3) & 3) + 8 * (r >> 5) + (r & 7);
+                    av[x] = a[(size_t)(128 * kb + r) * lda + i];
+                    bv[x] = b[(size_t)(128 * kb + r) * n + j];
+                }
+                const float p = fp8bs_model_mfma_dot128(av, bv);
+                acc = fmaf(p, as[(size_t)kb * lda + i] * bs[(size_t)kb * nb + j / 128], acc);
+            }
+            if (z == pieces - 1) own = acc; else part[z < 64 ? z : 63] = acc;
+        }
+        float total = own;
+        for (int z = 0; z + 1 < pieces && z < 64; z++) total += part[z];
+        if (out_f32) out_f32[t] = total;
+        if (out) out[t] = f32_to_bf16_rne(total);
+    }
+}
+
 /* `count` independent dot products: a, b are count x 128 codes in instruction order. */
 void fp8bs_model_mfma_dot128_batch(const uint8_t* a, const uint8_t* b, int count, float* out) {
     init_tables();

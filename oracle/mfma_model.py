@@ -108,6 +108,8 @@ def _lib():
         lib.fp8bs_model_gemm.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp, vp]
         lib.fp8bs_model_gemm_at.restype = None
         lib.fp8bs_model_gemm_at.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, vp, i32, vp, vp]
+        lib.fp8bs_model_gemm_at_segments.restype = None
+        lib.fp8bs_model_gemm_at_segments.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp, i32, vp, vp]
         lib._mfma_ready = True
     return lib
 
@@ -150,8 +152,48 @@ def model_kernel(data, split_k: int = 1, rows=None):
     return _bf16(out), torch.from_numpy(out32)
 
 
-def model_kernel_at(data, idx, split_k: int = 1):
-    """The same for selected elements: idx is an int array [count, 2] of (row, column); returns (bf16 [count], fp32 [count])."""
+class DealtKBlocks:
+    """How a call that deals K blocks, not tiles, to the workgroups (fp8bs_gemm_ex with split_k < 0) cuts the K
+    blocks of every tile.  The (tile, K block) pairs form one sequence - the tile_m x tile_n tiles in the band
+    order of the dense walk (bands of band_h tile rows, walked column by column), K ascending inside a tile - and
+    workgroup w of `grid` takes a run of total // grid pairs, the first total % grid runs one pair more."""
+
+    def __init__(self, m, n, k, tile_m, tile_n, grid, band_h=4):
+        self.tile_m, self.tile_n = tile_m, tile_n
+        tiles_m, tiles_n, kbt = -(-m // tile_m), -(-n // tile_n), k // 128
+        total = tiles_m * tiles_n * kbt
+        assert 1 <= grid <= total
+        q, r = divmod(total, grid)
+        starts = [w * q + min(w, r) for w in range(grid + 1)]
+        bounds, off = [], [0] * (tiles_m * tiles_n + 1)
+        order = []                                        # position in the sequence -> tile (tm, tn)
+        for band in range(-(-tiles_m // band_h)):
+            rows = min(band_h, tiles_m - band * band_h)
+            for tn in range(tiles_n):
+                for i in range(rows):
+                    order.append((band * band_h + i, tn))
+        cuts = {}
+        w = 0
+        for pos, (tm, tn) in enumerate(order):
+            x0 = pos * kbt
+            while starts[w] <= x0:
+                w += 1
+            inner, u = [], w
+            while starts[u] < x0 + kbt:
+                inner.append(starts[u] - x0)
+                u += 1
+            cuts[tm * tiles_n + tn] = [0] + inner + [kbt]
+        for t in range(tiles_m * tiles_n):
+            bounds += cuts[t]
+            off[t + 1] = len(bounds)
+        self.seg_off = np.asarray(off, dtype=np.int32)
+        self.seg_bounds = np.asarray(bounds, dtype=np.int32)
+        self.max_pieces = max(len(c) - 1 for c in cuts.values())
+
+
+def model_kernel_at(data, idx, split_k=1):
+    """The same for selected elements: idx is an int array [count, 2] of (row, column); returns (bf16 [count], fp32 [count]).
+    split_k: the K split, or a DealtKBlocks."""
     a, b, a_scale, b_scale = data[:4]
     m, k = a.shape
     n = b.shape[0]
@@ -159,6 +201,12 @@ def model_kernel_at(data, idx, split_k: int = 1):
     idx = np.ascontiguousarray(np.asarray(idx, dtype=np.int32).reshape(-1, 2))
     out = np.empty(idx.shape[0], dtype=np.uint16)
     out32 = np.empty(idx.shape[0], dtype=np.float32)
+    if isinstance(split_k, DealtKBlocks):
+        assert split_k.max_pieces <= 64
+        _lib().fp8bs_model_gemm_at_segments(sa.ctypes.data, sb.ctypes.data, ssa.ctypes.data, ssb.ctypes.data, m, n, k,
+                                            split_k.tile_m, split_k.tile_n, split_k.seg_off.ctypes.data, split_k.seg_bounds.ctypes.data,
+                                            idx.ctypes.data, idx.shape[0], out.ctypes.data, out32.ctypes.data)
+        return _bf16(out), torch.from_numpy(out32)
     _lib().fp8bs_model_gemm_at(sa.ctypes.data, sb.ctypes.data, ssa.ctypes.data, ssb.ctypes.data, m, n, k, split_k,
                                idx.ctypes.data, idx.shape[0], out.ctypes.data, out32.ctypes.data)
     return _bf16(out), torch.from_numpy(out32)

@@ -150,12 +150,48 @@ def measure(A: np.ndarray, B: np.ndarray, variant: int = 3, chunk: int = 2048) -
     return out
 
 
+def measure_16x16x32(A: np.ndarray, B: np.ndarray) -> np.ndarray:
+    """fp32 [count]: the same pairs through the FP8 MFMA of the reference's kernel, v_mfma_f32_16x16x32_fp8_fp8,
+    four chained per 128 k with the fp32 accumulator carried through
+    (1-amd-fp8-mm/amd-fp8-mm-submission.py:345-352), measured by the checker's probe kernel
+    (oracle/mfma_16x16x32_probe.hip)."""
+    from oracle import c_oracle
+    lib = c_oracle.load_probe()
+    dev = torch.device("cuda:0")
+    a = torch.from_numpy(np.ascontiguousarray(A)).to(dev)
+    b = torch.from_numpy(np.ascontiguousarray(B)).to(dev)
+    out = torch.zeros(A.shape[0], dtype=torch.float32, device=dev)
+    assert lib.mfma_probe_chain_16x16x32(a.data_ptr(), b.data_ptr(), A.shape[0], out.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def exact_sums(A: np.ndarray, B: np.ndarray) -> np.ndarray:
+    """float64 [count]: the exact value of every dot product (every product is a multiple of 2^-18 below 2^18,
+    so 128 of them add up without rounding in a double); NaN where an operand holds a NaN code."""
+    def dec(c):
+        c = c.astype(np.int64)
+        e, m = (c >> 3) & 15, c & 7
+        v = np.where(e == 0, m * 2.0 ** -9, (8 + m) * 2.0 ** (e - 10.0))
+        return np.where(c >> 7, -v, v)
+    s = (dec(A) * dec(B)).sum(axis=1)
+    nan = ((A & 0x7F) == 0x7F).any(axis=1) | ((B & 0x7F) == 0x7F).any(axis=1)
+    return np.where(nan, np.nan, s)
+
+
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--out", default=os.path.join(ROOT, "tests", "golden", "mfma_hw_vectors.npz"))
+    ap.add_argument("--out32", default=os.path.join(ROOT, "tests", "golden", "mfma_16x16x32_hw_vectors.npz"),
+                    help="results of the reference's instruction on the same vectors (D32 only; the codes are in --out)")
+    ap.add_argument("--only32", action="store_true", help="leave --out as it is")
     args = ap.parse_args()
     A, B, tags = vectors()
-    D = measure(A, B)
     os.makedirs(os.path.dirname(os.path.abspath(args.out)), exist_ok=True)
-    np.savez_compressed(args.out, A=A, B=B, D=D, tags=tags)
-    print("recorded %d dot products -> %s" % (len(D), args.out), flush=True)
+    if not args.only32:
+        D = measure(A, B)
+        np.savez_compressed(args.out, A=A, B=B, D=D, tags=tags)
+        print("recorded %d dot products -> %s" % (len(D), args.out), flush=True)
+    D32 = measure_16x16x32(A, B)
+    np.savez_compressed(args.out32, D32=D32)
+    print("recorded %d chained 16x16x32 results -> %s" % (len(D32), args.out32), flush=True)
