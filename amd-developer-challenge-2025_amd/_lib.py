@@ -93,8 +93,8 @@ _pycall = False
 
 def pycall():
     """The CPython binding of fp8bs_gemm_ex / fp8bs_gemm_grouped_ex (csrc/fp8bs_pycall.c: the same library
-    functions without ctypes' per-argument marshalling), or None where it has not been built; callers then use
-    the ctypes functions of load().  Either way the work is done by libfp8bs.so, which has no substitute."""
+    functions without ctypes' per-argument marshalling), or None where it has not been built or cannot be
+    imported (one warning); callers then use the ctypes functions of load().  Either way the work is done by libfp8bs.so, which has no substitute."""
     global _pycall
     if _pycall is False:
         load()                                        # the library must be there first; raises if it is not
@@ -103,11 +103,15 @@ def pycall():
         if os.path.exists(path):
             import importlib.machinery
             import importlib.util
-            loader = importlib.machinery.ExtensionFileLoader("_fp8bs_pycall", path)
-            spec = importlib.util.spec_from_file_location("_fp8bs_pycall", path, loader=loader)
-            mod = importlib.util.module_from_spec(spec)
-            loader.exec_module(mod)
-            _pycall = mod
+            try:
+                loader = importlib.machinery.ExtensionFileLoader("_fp8bs_pycall", path)
+                spec = importlib.util.spec_from_file_location("_fp8bs_pycall", path, loader=loader)
+                mod = importlib.util.module_from_spec(spec)
+                loader.exec_module(mod)
+                _pycall = mod
+            except (ImportError, OSError) as ex:      # built for another Python, or its libfp8bs.so cannot be resolved
+                import warnings
+                warnings.warn("_fp8bs_pycall.so cannot be imported (%s); binding libfp8bs.so through ctypes instead" % ex)
     return _pycall
 
 

@@ -229,11 +229,15 @@ bool vector_aligned(const void* a, const void* b, const void* c) {
 static __device__ __align__(256) unsigned char scratch[FP8BS_NOALLOC_SCRATCH_BYTES];
 static void* scratch_ptr[fp8bs::MAX_DEVICES];
 
-static int scratch_address(void** out) {
+static int scratch_address(void** out, hipStream_t stream) {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= fp8bs::MAX_DEVICES) return FP8BS_ERR_LAUNCH;
     void* p = __atomic_load_n(&scratch_ptr[dev], __ATOMIC_ACQUIRE);
     if (!p) {
+        // the lookup is no stream operation: it must not fall into a capture (the caller makes one eager call first)
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cap) != hipSuccess) { (void)hipGetLastError(); cap = hipStreamCaptureStatusNone; }
+        if (cap != hipStreamCaptureStatusNone) return FP8BS_ERR_CAPTURE;
         if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return FP8BS_ERR_LAUNCH;
         __atomic_store_n(&scratch_ptr[dev], p, __ATOMIC_RELEASE);     // the same value from every thread
     }
@@ -255,6 +259,7 @@ const char* fp8bs_strerror(int status) {
         case FP8BS_ERR_LAUNCH: return "kernel launch failed";
         case FP8BS_ERR_BAD_OFFSETS: return "grouped: num_experts must be positive";
         case FP8BS_ERR_BAD_VARIANT: return "unknown or inapplicable kernel variant";
+        case FP8BS_ERR_CAPTURE: return "fp8bs_gemm_noalloc: the first call on a device looks up the built-in scratch and must be made outside stream capture";
         case FP8BS_ERR_TIMEOUT: return "a workgroup gave up waiting for another workgroup's partial tile (status word of the workspace); the output of that call is not valid";
         case FP8BS_ERR_SCRATCH_LIMIT: return "fp8bs_gemm_noalloc: the K split planned for this shape needs more than the built-in scratch (FP8BS_NOALLOC_SCRATCH_BYTES); use fp8bs_gemm with a caller workspace";
         default: return "unknown fp8bs status";
@@ -264,6 +269,7 @@ const char* fp8bs_strerror(int status) {
 int fp8bs_plan(int m, int n, int k, int num_cus, fp8bs_plan_t* out) {
     if (!out) return FP8BS_ERR_NULL_POINTER;
     if (m <= 0 || n <= 0 || k <= 0 || (k % KBLK) != 0) return FP8BS_ERR_BAD_SHAPE;
+    if (num_cus <= 0) num_cus = fp8bs::device_cus();     // the current device's, 256 where there is none
     choose(m, n, k, num_cus, out);
     return FP8BS_OK;
 }
@@ -353,7 +359,7 @@ int fp8bs_gemm_noalloc(const void* a, const void* b, const float* a_scale, const
         if (plan.workspace_bytes > (uint64_t)FP8BS_NOALLOC_SCRATCH_BYTES) return FP8BS_ERR_SCRATCH_LIMIT;
     }
     void* ws = nullptr;
-    st = scratch_address(&ws);
+    st = scratch_address(&ws, (hipStream_t)stream);
     if (st != FP8BS_OK) return st;
     // Every partial element that the reduction reads is written by this call's main kernel first, so
     // nothing in the array has to start at zero.

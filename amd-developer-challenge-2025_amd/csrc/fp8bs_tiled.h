@@ -47,7 +47,7 @@ typedef unsigned short v4us __attribute__((ext_vector_type(4)));
 #define LDS_VOID(p) ((__attribute__((address_space(3))) void*)(p))
 
 static constexpr int KBLK = 128;  // scale block along K == K extent of one MFMA
-static constexpr int GROUP_TABLE_MAX = 128;   // grouped walk: up to 127 experts have their row ranges kept in LDS (2 KiB)
+static constexpr int GROUP_TABLE_MAX = 264;   // grouped walk: up to 263 experts have their row ranges kept in LDS (4.1 KiB)
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     v2f f = {lo, hi};
@@ -935,7 +935,13 @@ void gemm_tr_kernel(const GemmArgs p) {
         }
     } else {
         // bf16 through LDS so that the global stores are 16 bytes per lane and every store
-        // instruction writes whole rows of the wave tile (WNO*2 contiguous bytes each).  The last
+        // instruction writes whole rows of the wave tile (WNO*2 contiguous bytes each).  (Measured against the
+        // route through the registers alone - v_permlane16_swap pairing the 8-byte pieces of neighbouring lane
+        // groups into 16-byte ones, a rotation by 8 lanes so that an instruction writes 128-byte lines, no LDS:
+        // 4096^3 59.9-60.1 us against 60.2-60.5 with this staging on the same box, but 6144 x 7168 x 256 29.5
+        // against 27.5, 1024 x 7168 x 2048 19.4 against 18.9, the grouped configuration 915 against 901; with
+        // 64-byte pieces per row, no rotation, 58.1 against 56.1 on 4096^3.  Rows of 256 bytes per instruction
+        // are what the write path takes best, and the staging costs less than the narrower stores.)  The last
         // stage is free (after the barrier of the last K block no wave reads it and no copy into it is in
         // flight); the stages before it already receive the next tile.  Each wave stages its tile in two halves of
         // WM/2 rows in its own region; 16-byte chunks are XOR-swizzled by row so that neither the

@@ -14,7 +14,8 @@ from . import _lib
 from .submission import _check_operands, _is_kmajor, _stream_ptr
 
 
-_route_ws = {}     # device index -> uint8 tensor: the routing kernels' scratch, grown on demand, reused across calls
+_route_ws = {}     # (device index, stream) -> uint8 tensor: the routing kernels' scratch, grown on demand, reused across
+                   # calls on that stream (calls that overlap on two streams of one GPU must not share the count tables)
 
 
 def topk(scores: torch.Tensor, k: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -57,13 +58,19 @@ def route(top_idx: torch.Tensor, experts: int, out: Optional[Tuple[torch.Tensor,
                 raise ValueError("out: %s must be a contiguous int32 tensor of shape %s on top_idx's device" % (name, shape))
     lib = _lib.load()
     need = lib.fp8bs_moe_route_workspace_bytes(t, experts)
-    ws = _route_ws.get(dev.index)
-    if ws is None or ws.numel() < need:
-        ws = torch.empty(max(need, 4096), dtype=torch.uint8, device=dev)
-        _route_ws[dev.index] = ws
     with torch.cuda.device(dev):
+        stream = _stream_ptr(dev)
+        key = (dev.index, stream)
+        ws = _route_ws.get(key)
+        if ws is None or ws.numel() < need:
+            # A buffer that is outgrown stays alive until this stream's earlier kernels are done with it: the caching
+            # allocator hands a freed block only to later work of the stream it was allocated on.
+            if ws is None and len(_route_ws) >= 16:      # streams come and go: keep the table bounded (oldest entry out)
+                _route_ws.pop(next(iter(_route_ws)))
+            ws = torch.empty(max(need, 4096), dtype=torch.uint8, device=dev)
+            _route_ws[key] = ws
         _lib.check(lib.fp8bs_moe_route(top_idx.data_ptr(), t, experts, k, row_offsets.data_ptr(), row_map.data_ptr(),
-                                       slot_of.data_ptr(), ws.data_ptr(), ws.numel(), _stream_ptr(dev)))
+                                       slot_of.data_ptr(), ws.data_ptr(), ws.numel(), stream))
     return row_offsets, row_map, slot_of
 
 

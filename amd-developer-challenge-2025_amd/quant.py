@@ -26,11 +26,16 @@ def _check_input(x: torch.Tensor, name: str) -> None:
         raise ValueError("%s must be row-major (stride 1 along K), got strides %s" % (name, tuple(x.stride())))
 
 
-def quantize_a(x: torch.Tensor, row_map: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+def quantize_a(x: torch.Tensor, row_map: Optional[torch.Tensor] = None, fused: Optional[bool] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """x [T, K] -> (a e4m3fn [M, K] stride (1, M), a_scale fp32 [M, K/128] stride (1, M)).
 
     Without ``row_map`` M = T.  With ``row_map`` (int32 [M] on the GPU) output row i is input row
-    ``row_map[i]``: the expert-contiguous gather of routed tokens, fused into the quantiser.
+    ``row_map[i]``: the expert-contiguous gather of routed tokens.  Two routes, the same bytes: with at most as many
+    output rows as tokens the gather is fused into the quantiser (one kernel); with more (every token routed to
+    several experts, so rows repeat) every token is quantised once and the bytes are gathered by ``gather_a`` (two
+    kernels: 4096 -> 32768 rows x 7168 take 91-97 us that way against 154 us fused, which quantises each token once
+    per copy), provided the gather's fast path applies (T and M multiples of 4, T <= 40960).  ``fused`` = True / False
+    forces the one-kernel / two-kernel route.
     """
     _check_input(x, "x")
     t, k = x.shape
@@ -38,6 +43,10 @@ def quantize_a(x: torch.Tensor, row_map: Optional[torch.Tensor] = None) -> Tuple
         if row_map.dtype != torch.int32 or row_map.dim() != 1 or row_map.device != x.device or not row_map.is_contiguous():
             raise ValueError("row_map must be a contiguous int32 vector on x's device")
         m = row_map.numel()
+        if fused is None:
+            fused = not (m > t and t % 4 == 0 and m % 4 == 0 and 0 < t <= 40960)
+        if not fused:
+            return gather_a(*quantize_a(x), row_map)
     else:
         m = t
     a_store = torch.empty(k, m, dtype=torch.float8_e4m3fn, device=x.device)

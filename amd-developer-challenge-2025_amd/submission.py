@@ -119,7 +119,8 @@ def _check_operands(a, b, a_scale, b_scale, c, rows, n, k):
 
 
 def plan(m: int, n: int, k: int) -> _lib.Plan:
-    """The kernel variant, split-K and grid the library would choose for a dense shape (host only)."""
+    """The kernel variant, split-K and grid the library would choose for a dense shape (host only).
+    num_cus = 0: the library asks the current device for its CU count, as fp8bs_gemm does (256 without a GPU)."""
     p = _lib.Plan()
     _lib.check(_lib.load().fp8bs_plan(m, n, k, 0, ctypes.byref(p)))
     return p

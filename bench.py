@@ -33,10 +33,22 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP8_TFLOPS = 5033.0      # 256 CU x 2.4 GHz x 8192 FLOP/clk/CU, dense e4m3
 PEAK_HBM_GBS = 8000.0
-# HBM/fabric bytes per launch of the 256x256 kernel on configuration 2, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (KiB per dispatch: 49,770 and 32,770) scaled by what the same counters read for a 128 MiB
-# device copy (`--calibrate-copy`: x2.00 and x1.00); the summary is profiles/gemm_tr_256x256_cfg2_4096cubed.txt
-TRAFFIC_CFG2_BYTES = (49779 * 2.00 + 32783 * 1.00) * 1024
+# HBM/fabric bytes per launch of the 256x256 kernel on configuration 2: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB
+# per dispatch), each scaled by what the same counter reads for a 128 MiB device copy (`--calibrate-copy`).  The figures
+# live beside the profile summary they come from, together with the kernel-trace durations of the same command.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemm_tr_256x256_cfg2_4096cubed.traffic.json")
+
+
+def profiled_traffic():
+    """(bytes per launch or None, the profile's record) from TRAFFIC_FILE; (None, {}) when it is missing."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)
+        traffic = (rec["fetch_size_kib_per_dispatch"] * rec["fetch_scale_from_128MiB_copy"]
+                   + rec["write_size_kib_per_dispatch"] * rec["write_scale_from_128MiB_copy"]) * 1024
+        return traffic, rec
+    except (OSError, KeyError, ValueError):
+        return None, {}
 
 
 def algorithmic_bytes(m, n, k):
@@ -310,6 +322,10 @@ def main():
     us_sustained = statistics.median(per_call)
     achieved = flops / (us_sustained * 1e-6) / 1e12
     plan = pkg.plan(cfg2.m, cfg2.n, cfg2.k)
+    traffic, prof = profiled_traffic()
+    # only when the planned kernel is the profiled one do the profile's figures belong on this line
+    if pkg._lib.VARIANT_NAMES.get(plan.variant) != "t256x256" or plan.split_k != 1 or plan.stream_k != 0:
+        traffic, prof = None, {}
 
     result = {
         "metric": "TFLOP/s (FP8 block-scaled GEMM, 2*M*N*K per call)", "value": round(value, 2), "unit": "TFLOP/s",
@@ -317,13 +333,22 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3fn x fp8_e4m3fn -> f32 -> bf16",
         "data": "synthetic",
         "config": {"workload": "cfg2: M=N=K=4096, A 1x128 / B 128x128 fp32 block scales, bf16 out, seed %d" % cfg2.seed,
-                   "variant": pkg._lib.VARIANT_NAMES[plan.variant], "split_k": plan.split_k, "grid": plan.grid_x,
+                   "variant": pkg._lib.VARIANT_NAMES.get(plan.variant, "variant %d" % plan.variant), "split_k": plan.split_k, "grid": plan.grid_x,
                    "preheat_calls": preheated},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_FP8_TFLOPS, 4), "traffic": TRAFFIC_CFG2_BYTES,
+                     "frac": round(achieved / PEAK_FP8_TFLOPS, 4), "traffic": traffic,
                      "us_per_launch": round(us_sustained, 3), "us_sustained": round(us_sustained, 3),
                      "us_sustained_min_max": [round(min(per_call), 3), round(max(per_call), 3)], "us_burst": round(us_burst, 3)},
     }
+    if prof.get("trace_average_us"):
+        # the committed rocprofv3 --kernel-trace figures of the same command, and why they sit above back-to-back launches
+        t_avg = prof["trace_average_us"]
+        result["roofline"]["profile"] = {
+            "trace_average_us": t_avg, "trace_median_us": prof.get("trace_median_us"),
+            "hip_events_in_the_traced_run_us": prof.get("hip_events_in_the_traced_run_us"),
+            "frac_from_trace_average": round(flops / (t_avg * 1e-6) / 1e12 / PEAK_FP8_TFLOPS, 4),
+            "differs_from_us_sustained_by": round(t_avg / us_sustained - 1.0, 4),
+            "reason": prof.get("trace_note"), "summary": prof.get("summary")}
 
     # ---- other configurations ----
     per_config = {}
@@ -404,7 +429,7 @@ def main():
                                                      "kernels": 3, "note": "top-k + count + assign (scan fused), no host sync; mostly the Python wrapper's allocations"}
         row_map = moe.route(moe.topk(scores, cfg5.topk), cfg5.experts)[1]
         x = torch.randn(cfg5.m, cfg5.k, generator=g, device=dev)
-        us, us_min = time_calls(lambda i: quant.quantize_a(x, row_map), max(args.steps // 2, 5), 3)
+        us, us_min = time_calls(lambda i: quant.quantize_a(x, row_map, fused=True), max(args.steps // 2, 5), 3)
         rows = row_map.numel()
         by = cfg5.m * cfg5.k * 4 + rows * cfg5.k + 4 * rows * (cfg5.k // 128)
         per_config["quant_a_gather_fp32_4096to32768x7168"] = {
@@ -480,7 +505,15 @@ def main():
         per_config["leaderboard_18_shapes"] = {
             "geomean_us": round(geo, 2), "mean_us": round(sum(r["us"] for r in rows_) / len(rows_), 2),
             "shapes": ["%dx%dx%d: %.1f us, %.0f TF" % (r["m"], r["n"], r["k"], r["us"], r["tflops"]) for r in rows_]}
-    result["per_config"] = per_config
+    # the headline metric's two aggregates: geometric mean of the MFMA fractions of configurations 2, 3 and 5, and the
+    # HBM fraction of configuration 4 (present when those configurations were run)
+    summary = {}
+    if "cfg3" in per_config and "cfg5" in per_config:
+        fr = [result["roofline"]["frac"], per_config["cfg3"]["frac"], per_config["cfg5"]["frac"]]
+        summary["geomean_frac_cfg2_3_5"] = round((fr[0] * fr[1] * fr[2]) ** (1.0 / 3.0), 4)
+    if "cfg4" in per_config:
+        summary["cfg4_hbm_frac"] = per_config["cfg4"]["frac"]
+    result["per_config"] = dict(summary, **per_config)
 
     # ---- CPU baseline: the oracle on the same configuration-2 inputs, host cores ----
     if not args.no_cpu_baseline:

@@ -41,9 +41,10 @@ enum {
     FP8BS_ERR_BAD_VARIANT = 7,    /* forced variant id unknown or not applicable             */
     FP8BS_ERR_SCRATCH_LIMIT = 8,  /* fp8bs_gemm_noalloc: the shape's K split needs more than
                                      FP8BS_NOALLOC_SCRATCH_BYTES of partial planes            */
-    FP8BS_ERR_TIMEOUT = 9         /* never returned by a call (calls do not wait for the GPU): the value a
+    FP8BS_ERR_TIMEOUT = 9,        /* never returned by a call (calls do not wait for the GPU): the value a
                                      kernel leaves in the first word of the workspace when a workgroup's
                                      bounded wait for another workgroup's partial tile gave up     */
+    FP8BS_ERR_CAPTURE = 10        /* fp8bs_gemm_noalloc: first call on this device made under stream capture */
 };
 
 /* Kernel variants the planner chooses from. */
@@ -86,7 +87,8 @@ int fp8bs_version(void);
 const char* fp8bs_strerror(int status);
 
 /* Host-only planning: no GPU needed. Replaces the dispatch of
- * 1-amd-fp8-mm/amd-fp8-mm-submission.py:528-578. `num_cus` <= 0 means 256 (MI355X).  The plan is the one
+ * 1-amd-fp8-mm/amd-fp8-mm-submission.py:528-578. `num_cus` <= 0 means the CU count of the current device, as fp8bs_gemm, fp8bs_gemm_noalloc and
+ * fp8bs_workspace_bytes use it (256, MI355X's, where no device can be asked).  The plan is the one
  * fp8bs_gemm follows with a workspace of workspace_bytes; without the workspace of a planned K split
  * fp8bs_gemm runs the best plan that needs none (slower, same result up to the summation order). */
 int fp8bs_plan(int m, int n, int k, int num_cus, fp8bs_plan_t* out);
@@ -123,7 +125,11 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
  * A shape whose planned K split needs more partial-plane bytes than that returns FP8BS_ERR_SCRATCH_LIMIT
  * and launches nothing.  All calls on one GPU share the one array: calls that overlap on a GPU (two
  * streams, two threads) race on it; calls on one stream are ordered and safe.  Nothing in the array has to
- * be cleared between calls (every partial element read was written by the same call). */
+ * be cleared between calls (every partial element read was written by the same call).
+ * Under HIP graph capture: make one eager call per device and shape first.  The first call on a device looks the
+ * array's address up (hipGetSymbolAddress) and the first launch of every kernel instantiation raises that kernel's
+ * dynamic-LDS limit (hipFuncSetAttribute); neither is a stream operation that a capture could record.  A first
+ * call that finds its stream capturing returns FP8BS_ERR_CAPTURE and launches nothing. */
 #define FP8BS_NOALLOC_SCRATCH_BYTES (32u * 1024u * 1024u)
 int fp8bs_gemm_noalloc(const void* a, const void* b, const float* a_scale, const float* b_scale,
                        void* c, int m, int n, int k, void* stream);

@@ -26,6 +26,27 @@ def test_library_exports_every_declared_symbol(pkg):
     assert lib.fp8bs_version() >= 100
 
 
+def test_every_variant_has_a_name_and_the_plan_struct_matches_the_header(pkg):
+    text = open(os.path.join(ROOT, "include", "fp8bs.h")).read()
+    count = int(re.search(r"FP8BS_VARIANT_COUNT\s*=\s*(\d+)", text).group(1))
+    assert set(pkg._lib.VARIANT_NAMES) == set(range(count))
+    body = re.search(r"typedef struct fp8bs_plan_t \{(.*?)\} fp8bs_plan_t;", text, flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = [f.strip() for decl in re.findall(r"(?:int32_t|uint64_t)\s+([^;]+);", body) for f in decl.split(",")]
+    assert fields == [name for name, _ in pkg._lib.Plan._fields_]
+
+
+def test_plan_with_the_devices_cu_count(pkg):
+    """num_cus <= 0 asks the current device (256 where there is none), the count fp8bs_gemm plans with."""
+    lib = pkg._lib.load()
+    a, b = pkg._lib.Plan(), pkg._lib.Plan()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count if torch.cuda.is_available() else 256
+    for shape in ((4096, 2112, 7168), (64, 18432, 7168), (1024, 512, 7168)):
+        assert lib.fp8bs_plan(*shape, 0, ctypes.byref(a)) == 0 and lib.fp8bs_plan(*shape, cus, ctypes.byref(b)) == 0
+        assert bytes(a) == bytes(b)
+        assert a.stream_k == 0 and a.workspace_bytes == pkg.workspace_bytes(*shape)
+
+
 def test_plan_shape_families(pkg):
     p = pkg.plan(4096, 4096, 4096)
     assert p.variant == 2 and (p.tile_m, p.tile_n) == (256, 256) and p.split_k == 1 and p.workspace_bytes == 0

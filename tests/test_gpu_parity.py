@@ -404,10 +404,11 @@ def test_grouped_small(pkg, oracle, dev, tokens, n, k, experts, topk):
 @pytest.mark.parametrize("variant", [0, 3, 11, 12])
 @pytest.mark.parametrize("tokens,n,k,experts,topk", [(200, 256, 256, 70, 3), (500, 136, 128, 127, 2), (500, 136, 128, 128, 2),
                                                       (300, 256, 128, 200, 4), (2048, 512, 256, 3, 2), (6000, 256, 128, 2, 1),
-                                                      (3000, 384, 128, 9, 1)])
+                                                      (3000, 384, 128, 9, 1), (4096, 256, 256, 256, 8), (1000, 136, 128, 263, 2),
+                                                      (1000, 136, 128, 264, 2), (900, 256, 128, 400, 3)])
 def test_grouped_expert_counts_and_tile_orders(pkg, oracle, dev, variant, tokens, n, k, experts, topk):
-    """The walk's two ways of finding a tile's expert - the table in LDS (fewer than 128 experts; more than 64
-    take two rounds of it) and the loop over row_offsets - and its two orders of the tiles (across the experts
+    """The walk's two ways of finding a tile's expert - the table in LDS (up to 263 experts, 256 among them; more
+    than 64 take several rounds of it) and the loop over row_offsets (264 experts and more) - and its two orders of the tiles (across the experts
     when they hold less than a tile of rows on average, expert by expert otherwise, experts of more than eight
     tile rows cut into bands): every element against the oracle, no row left unwritten."""
     cpu = pkg.inputs.make_grouped(pkg.inputs.CONFIGS[4], tokens=tokens, n=n, k=k, experts=experts, topk=topk)

@@ -129,10 +129,12 @@ def test_gather_after_quantise_equals_fused_gather(quant, dev):
     g = torch.Generator().manual_seed(77)
     x = (torch.randn(4096, 7168, generator=g) * 3).to(dev)
     row_map = torch.randint(0, 4096, (32768,), dtype=torch.int32, generator=g).to(dev)
-    a1, s1 = quant.quantize_a(x, row_map)
+    a1, s1 = quant.quantize_a(x, row_map, fused=True)
     a2, s2 = quant.gather_a(*quant.quantize_a(x), row_map)
     assert a2.shape == a1.shape and a2.stride() == a1.stride() and s2.stride() == s1.stride()
     assert torch.equal(a1.view(torch.uint8), a2.view(torch.uint8)) and torch.equal(s1, s2)
+    a3, s3 = quant.quantize_a(x, row_map)                        # more rows than tokens: the two-kernel route by default
+    assert torch.equal(a1.view(torch.uint8), a3.view(torch.uint8)) and torch.equal(s1, s3) and a3.stride() == a1.stride()
 
 
 def test_gather_a_argument_errors(quant, dev):

@@ -165,3 +165,28 @@ def test_scores_to_grouped_gemm_chain(moe, quant, pkg, oracle, ro, dev):
                               torch.zeros(rows, n, dtype=torch.bfloat16)))
     ok, nbad, maxerr = oracle.within_tolerance(out.cpu(), ref, 2e-2, 1e-3)
     assert ok, "%d outside the bar, max err %g" % (nbad, maxerr)
+
+
+def test_routing_calls_that_overlap_on_two_streams(pkg, dev):
+    """moe.route keeps one scratch buffer per device and stream: two different routing problems issued
+    alternately on two streams, without waiting in between, each give their serial result (one buffer shared by
+    both streams would let one call's count tables overwrite the other's)."""
+    moe = importlib.import_module("amd-developer-challenge-2025_amd.moe")
+    probs = []
+    for tokens, experts, k, seed in ((4096, 32, 8, 1), (3000, 48, 6, 2)):
+        g = torch.Generator(device=dev).manual_seed(seed)
+        idx = moe.topk(torch.rand(tokens, experts, generator=g, device=dev), k)
+        serial = tuple(t.clone() for t in moe.route(idx, experts))
+        probs.append((idx, experts, serial))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[], []]
+    for rep in range(20):
+        for i, (idx, experts, _) in enumerate(probs):
+            with torch.cuda.stream(streams[i]):
+                outs[i].append(moe.route(idx, experts))
+    torch.cuda.synchronize()
+    for i, (_, _, serial) in enumerate(probs):
+        for rep, got in enumerate(outs[i]):
+            for name, x, y in zip(("row_offsets", "row_map", "slot_of"), got, serial):
+                assert torch.equal(x, y), "stream %d call %d: %s" % (i, rep, name)
