@@ -56,21 +56,21 @@ def test_plan_shape_families(pkg):
     assert p.block_threads == 512 and p.lds_bytes == 3 * (128 * 320 + 1024 + 256)
     assert p.workspace_bytes == p.split_k * 64 * 18432 * 4 == pkg.workspace_bytes(64, 18432, 7168)
     p = pkg.plan(130, 190, 256)                         # n not a multiple of 8, short K -> a tiled kernel without a K split
-    assert p.variant in (2, 3, 4, 9, 10, 11) and p.split_k == 1
+    assert p.variant in (2, 3, 4, 9, 10, 11, 12) and p.split_k == 1
     p, q = pkg.plan(1024, 190, 7168), pkg.plan(1024, 192, 7168)   # long K, few tiles: a K split, also with n off the 8-column grid
-    assert p.variant == q.variant and p.variant in (2, 3, 4, 9, 10, 11) and p.split_k == q.split_k > 1
+    assert p.variant == q.variant and p.variant in (2, 3, 4, 9, 10, 11, 12) and p.split_k == q.split_k > 1
     assert p.workspace_bytes == p.split_k * 1024 * 190 * 4
     for m in (130, 4095, 3, 1):                               # any m: the tiled kernels, one launch, nothing extra in the workspace
         p, q = pkg.plan(m, 192, 256), pkg.plan((m + 3) & ~3, 192, 256)
-        assert p.variant == q.variant and p.variant not in (1, 6, 7, 8, 12) and p.split_k == q.split_k
+        assert p.variant == q.variant and p.variant not in (1, 6, 7, 8) and p.split_k == q.split_k
         assert p.workspace_bytes == (p.split_k * m * 192 * 4 if p.split_k > 1 else 0)
     p, q = pkg.plan(3, 18432, 7168), pkg.plan(4, 18432, 7168) # a few rows against a large b: the same skinny plan for any m
     assert p.variant == q.variant == 12 and p.split_k == q.split_k and p.workspace_bytes == p.split_k * 3 * 18432 * 4
-    assert pkg.plan(3, 190, 256).variant in (3, 4)
+    assert pkg.plan(3, 190, 256).variant in (3, 4, 12)
     p = pkg.plan(256, 512, 1024)                        # small: one of the sub-256 tiles, never the scalar kernel
-    assert p.variant in (3, 4, 10) and p.split_k >= 1 and p.split_k <= 8
+    assert p.variant in (3, 4, 10, 12) and p.split_k >= 1 and p.split_k <= 8
     p = pkg.plan(1024, 512, 7168)                       # few tiles, long K: the planner splits K
-    assert p.variant in (3, 4, 10) and p.split_k > 1
+    assert p.variant in (3, 4, 10, 12) and p.split_k > 1
     p = pkg.plan(6144, 4608, 7168)                      # large: the 256x256 tile, no split
     assert p.variant == 2 and p.split_k == 1
     p = pkg.plan(4096, 2112, 7168)                      # 2112 = 11 x 192: 242 tiles of 192x192 instead of 144 of 256x256, 16 of them a quarter full
@@ -81,20 +81,20 @@ def test_plan_shape_families(pkg):
     assert p.variant == 10 and (p.tile_m, p.tile_n) == (256, 128) and p.lds_bytes == 3 * (128 * 384 + 1024 + 256)
 
 
-def test_plan_skinny_tile_only_for_few_rows_against_a_large_b(pkg):
-    """The 64x256 three-stage tile is planned for at most 64 rows and a B of 24 MB or more; everything else goes
-    through the cost model of the other tiles (more rows would make it copy B twice).  The streaming kernels are
-    never planned (forced variants only)."""
+def test_plan_skinny_rule_and_the_streaming_kernels(pkg):
+    """At most 64 rows against a B of 24 MB or more: always the 64x256 three-stage tile, with the K split of the
+    streaming model.  Everything else goes through the cost model of all the tiles (the 64x256 tile among them).
+    The streaming kernels are never planned (forced variants only)."""
     for m, n, k, skinny in [(64, 18432, 7168, True), (16, 18432, 7168, True), (4, 18432, 7168, True), (64, 7168, 7168, True),
                             (1, 28672, 4096, True), (64, 18440, 7168, True), (63, 18429, 7168, True),
                             (65, 18432, 7168, False), (128, 18432, 7168, False), (64, 2048, 7168, False),
-                            (64, 7168, 2048, False), (32, 512, 2048, False)]:
+                            (64, 7168, 2048, False), (32, 512, 2048, False), (1536, 1536, 4096, False)]:
         p = pkg.plan(m, n, k)
-        assert (p.variant == 12) == skinny, (m, n, k, p.variant)
+        if skinny:
+            assert p.variant == 12 and p.grid_x == -(-n // 256) * p.split_k, (m, n, k, p.variant)
         assert p.variant not in (1, 6, 7, 8)
         assert 1 <= p.split_k <= 8 and p.workspace_bytes == (p.split_k * m * n * 4 if p.split_k > 1 else 0)
-        if skinny:
-            assert p.grid_x == -(-n // 256) * p.split_k
+    assert pkg.plan(1536, 1536, 4096).variant == 12           # the cost model's pick for a few hundred rows per tile column
     for m in (1, 5, 63):                                      # rows that are not a multiple of four: the same plan
         p, q = pkg.plan(m, 18432, 7168), pkg.plan((m + 3) & ~3, 18432, 7168)
         assert p.variant == q.variant == 12 and p.split_k == q.split_k
