@@ -3,6 +3,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs 2,3,4,5] [--no-cpu-baseline]
     python bench.py --mfma-ceiling        (what the matrix cores reach without the GEMM's schedule)
     python bench.py --calibrate-copy      (yardstick for rocprofv3's FETCH_SIZE / WRITE_SIZE)
+    python bench.py --only CFG:VARIANT:SPLIT   (one dense configuration with the tile and K split forced; SPLIT < 0 deals
+                                           K blocks to the workgroups in one launch: what the profiles of that mode run)
 
 A step is one call of custom_kernel on configuration 2 (M=N=K=4096, the configuration the headline
 metric is quoted on) with inputs resident in HBM.  W untimed warm-up steps and an untimed pre-heat (calls
@@ -251,6 +253,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run plain device copies of a known size (128 MiB read + 128 MiB written per copy), "
                          "the yardstick for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--only", type=str, default="",
+                    help="CFG:VARIANT:SPLIT - time only dense configuration CFG (2, 3 or 4) with the kernel variant and K split "
+                         "forced (SPLIT < 0: K blocks dealt to the workgroups, one launch); rotating input sets for the HBM-bound one")
     ap.add_argument("--mfma-ceiling", action="store_true",
                     help="only time the library's measurement kernel: the FP8 MFMA stream of the 256x256 tile in a "
                          "register-only loop, alone and with the fold / the transposing LDS reads / the global->LDS copies "
@@ -276,6 +281,20 @@ def main():
         return
     if args.mfma_ceiling:
         print(json.dumps({"mfma_ceiling": mfma_ceiling(pkg, dev)}))
+        return
+    if args.only:
+        idx, variant, split = (int(x) for x in args.only.split(":"))
+        cfg = pkg.inputs.CONFIGS[idx - 1]
+        by = algorithmic_bytes(cfg.m, cfg.n, cfg.k)
+        fl = 2.0 * cfg.m * cfg.n * cfg.k
+        hbm = fl / by < 629
+        nsets = min(8, -(-3 * 256 * 2 ** 20 // by)) if hbm else 1
+        sets = [gpu_dense_inputs(pkg, cfg, dev, cfg.seed + 100 * s) for s in range(nsets)]
+        us, us_min = time_calls(lambda i: pkg.custom_kernel(sets[i % nsets], variant=variant, split_k=split), args.steps, args.warmup)
+        print(json.dumps({"only": {"config": cfg.name, "variant": pkg._lib.VARIANT_NAMES.get(variant, str(variant)), "split_k": split,
+                                   "input_sets": nsets, "us": round(us, 2), "us_min": round(us_min, 2),
+                                   "frac": round(by / us * 1e-3 / PEAK_HBM_GBS if hbm else fl / us * 1e-6 / PEAK_FP8_TFLOPS, 4),
+                                   "bound": "hbm" if hbm else "mfma"}}))
         return
     cfg2 = pkg.inputs.CONFIGS[1]
 
