@@ -111,7 +111,21 @@ int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* 
 
 /* Same as fp8bs_gemm with the variant and split-K forced (testing and benchmarking the shape
  * families against each other). variant = FP8BS_VARIANT_AUTO and split_k = 0 reproduce fp8bs_gemm.
- * Workspace requirement for a forced split_k > 1: split_k * m * n * 4 bytes. */
+ * Workspace requirement for a forced split_k > 1: split_k * m * n * 4 bytes.
+ * split_k < 0: the K split in ONE launch - the role of the reference's split kernel plus merge kernel
+ * (1-amd-fp8-mm/amd-fp8-mm-submission.py:371-511) without the second launch.  K blocks, not tiles, are dealt to
+ * the workgroups (one per place on the chip, G = min(places, tiles * K/128); the tiled variants only, else
+ * FP8BS_ERR_BAD_VARIANT); a workgroup whose run of K blocks ends inside a tile leaves an fp32 partial tile in the
+ * workspace and raises a flag there, the workgroup that holds the tile's last K block waits for the flags (a
+ * bounded number of polls), adds the partial tiles in ascending K to its own accumulators - a fixed order, so the
+ * result is the same from run to run - and writes c.  Workspace: 16384 + G * tile_m * tile_n * 4 bytes
+ * (FP8BS_ERR_WORKSPACE if smaller; at most 64 MiB + 16 KiB on 256 CUs), contents unspecified on entry, one
+ * call at a time per workspace.  Its first word is a status: a wait that gives up stores FP8BS_ERR_TIMEOUT there
+ * and the kernel still runs to its end (c is then not valid); nothing else ever writes that word, so a caller
+ * that means to read it zeroes it once after allocating.  The environment variable FP8BS_STREAMK_SPIN, read once,
+ * sets the polls per flag (default 262144, about a quarter of a second; negative: every wait gives up at once).
+ * Measured on MI355X this form is not faster than the planned K split with its reduce launch, so fp8bs_plan
+ * never chooses it (stream_k of a plan is 0). */
 int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale,
                   void* c, void* ws, size_t ws_bytes, int m, int n, int k,
                   int variant, int split_k, void* stream);
