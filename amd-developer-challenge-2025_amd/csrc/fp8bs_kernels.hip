@@ -260,16 +260,33 @@ void gemm_skinny_kernel(const GemmArgs p) {
 // arrays of m*n elements, so the row length plays no part.  VEC: m*n is a multiple of 8 and c starts on a
 // 16-byte boundary; otherwise the same sums, element by element, with the last group cut at m*n.
 // ---------------------------------------------------------------------------------------------------
-template <bool VEC>
+// SPLIT > 0: the number of planes is a compile-time fact, so all of a thread's loads are issued before the first add
+// (with a run-time count the compiler keeps the loop and every plane's load waits for the previous plane's add: the
+// kernel then takes one memory latency per plane); SPLIT == 0: any count.  The sum is taken in ascending order of
+// the planes either way.
+template <bool VEC, int SPLIT>
 __global__ __launch_bounds__(256)
 void splitk_reduce_kernel(const float* __restrict__ ws, uint16_t* __restrict__ c, size_t mn, int split_k) {
     size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 8;
     if (i >= mn) return;
     if constexpr (VEC) {
-        v4f s0 = *(const v4f*)(ws + i), s1 = *(const v4f*)(ws + i + 4);
-        for (int z = 1; z < split_k; z++) {
-            s0 += *(const v4f*)(ws + (size_t)z * mn + i);
-            s1 += *(const v4f*)(ws + (size_t)z * mn + i + 4);
+        v4f s0, s1;
+        if constexpr (SPLIT > 0) {
+            v4f p0[SPLIT], p1[SPLIT];
+#pragma unroll
+            for (int z = 0; z < SPLIT; z++) {
+                p0[z] = __builtin_nontemporal_load((const v4f*)(ws + (size_t)z * mn + i));
+                p1[z] = __builtin_nontemporal_load((const v4f*)(ws + (size_t)z * mn + i + 4));
+            }
+            s0 = p0[0]; s1 = p1[0];
+#pragma unroll
+            for (int z = 1; z < SPLIT; z++) { s0 += p0[z]; s1 += p1[z]; }
+        } else {
+            s0 = *(const v4f*)(ws + i); s1 = *(const v4f*)(ws + i + 4);
+            for (int z = 1; z < split_k; z++) {
+                s0 += *(const v4f*)(ws + (size_t)z * mn + i);
+                s1 += *(const v4f*)(ws + (size_t)z * mn + i + 4);
+            }
         }
         v4i o;
         o[0] = (int)pack_bf16x2(s0[0], s0[1]); o[1] = (int)pack_bf16x2(s0[2], s0[3]);
@@ -391,10 +408,22 @@ hipError_t launch_gemm(int variant, int mode, const GemmArgs& a, hipStream_t str
 hipError_t launch_splitk_reduce(const float* ws, uint16_t* c, size_t mn, int split_k, hipStream_t stream) {
     size_t threads = (mn + 7) / 8;
     unsigned blocks = (unsigned)((threads + 255) / 256);
-    if ((mn & 7) == 0 && ((uintptr_t)c & 15) == 0 && ((uintptr_t)ws & 15) == 0)
-        hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3(blocks), dim3(256), 0, stream, ws, c, mn, split_k);
-    else
-        hipLaunchKernelGGL(splitk_reduce_kernel<false>, dim3(blocks), dim3(256), 0, stream, ws, c, mn, split_k);
+    if ((mn & 7) == 0 && ((uintptr_t)c & 15) == 0 && ((uintptr_t)ws & 15) == 0) {
+        void (*kern)(const float*, uint16_t*, size_t, int) = splitk_reduce_kernel<true, 0>;
+        switch (split_k) {
+            case 2: kern = splitk_reduce_kernel<true, 2>; break;
+            case 3: kern = splitk_reduce_kernel<true, 3>; break;
+            case 4: kern = splitk_reduce_kernel<true, 4>; break;
+            case 5: kern = splitk_reduce_kernel<true, 5>; break;
+            case 6: kern = splitk_reduce_kernel<true, 6>; break;
+            case 7: kern = splitk_reduce_kernel<true, 7>; break;
+            case 8: kern = splitk_reduce_kernel<true, 8>; break;
+            default: break;
+        }
+        hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), 0, stream, ws, c, mn, split_k);
+    } else {
+        hipLaunchKernelGGL((splitk_reduce_kernel<false, 0>), dim3(blocks), dim3(256), 0, stream, ws, c, mn, split_k);
+    }
     return hipGetLastError();
 }
 
