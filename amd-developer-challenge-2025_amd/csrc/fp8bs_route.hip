@@ -239,15 +239,28 @@ void moe_combine_kernel(const uint16_t* __restrict__ y, const int32_t* __restric
     const int t = blockIdx.x;
     for (int c = threadIdx.x * 8; c < d; c += RB * 8) {
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int j = 0; j < topk; j++) {
-            const int slot = slot_of[(size_t)t * topk + j];
-            if (slot < 0 || slot >= rows) continue;
-            const float w = weights[(size_t)t * topk + j];
-            const cv4i v = *(const cv4i*)(y + (size_t)slot * d + c);
+        // four rows at a time, all four loads issued before the first is used (one after the other a step costs
+        // one memory latency per choice); a choice that is skipped enters as weight 0 times zeros, which leaves
+        // the sum as it is
+        for (int j0 = 0; j0 < topk; j0 += 4) {
+            cv4i v[4];
+            float w[4];
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                acc[2 * i] = __builtin_fmaf(w, __builtin_bit_cast(float, (uint32_t)v[i] << 16), acc[2 * i]);
-                acc[2 * i + 1] = __builtin_fmaf(w, __builtin_bit_cast(float, (uint32_t)v[i] & 0xFFFF0000u), acc[2 * i + 1]);
+                const int j = j0 + i;
+                const int slot = j < topk ? slot_of[(size_t)t * topk + j] : -1;
+                const bool ok = slot >= 0 && slot < rows;
+                w[i] = ok ? weights[(size_t)t * topk + j] : 0.f;
+                v[i] = (cv4i){0, 0, 0, 0};
+                if (ok) v[i] = __builtin_nontemporal_load((const cv4i*)(y + (size_t)slot * d + c));
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+#pragma unroll
+                for (int x = 0; x < 4; x++) {
+                    acc[2 * x] = __builtin_fmaf(w[i], __builtin_bit_cast(float, (uint32_t)v[i][x] << 16), acc[2 * x]);
+                    acc[2 * x + 1] = __builtin_fmaf(w[i], __builtin_bit_cast(float, (uint32_t)v[i][x] & 0xFFFF0000u), acc[2 * x + 1]);
+                }
             }
         }
         cv4i o;
