@@ -209,3 +209,49 @@ def test_model_kernel_on_the_exact_fixture_and_against_the_oracle(mm, oracle, go
     assert torch.equal(at.view(torch.int16), mod[idx[:, 0], idx[:, 1]].view(torch.int16))
     rows, _ = mm.model_kernel(cfg1, rows=(100, 108))
     assert torch.equal(rows.view(torch.int16), mod[100:108].view(torch.int16))
+
+
+def test_dealt_k_blocks_partition_and_the_model_of_its_sums(mm, golden_gemm):
+    """DealtKBlocks restates how a call that deals K blocks to the workgroups cuts every tile: the runs are
+    contiguous, differ by at most one pair, cover every (tile, K block) pair once, and a run that is longer than
+    a tile holds whole tiles.  On the exact power-of-two fixture any order of the partial sums gives the exact
+    bits, so the modelled call must reproduce the fixture whatever the cuts (a wrong tile or K-block index in the
+    restatement would not)."""
+    for (m, n, k, tm, tn, grid) in ((4096, 2112, 7168, 256, 256, 256), (64, 18432, 7168, 64, 256, 256), (256, 512, 1024, 128, 128, 32),
+                                    (1000, 520, 1024, 64, 128, 768), (300, 200, 128, 256, 256, 2), (4096, 4096, 512, 256, 256, 256)):
+        tiles, kbt = -(-m // tm) * -(-n // tn), k // 128
+        grid = min(grid, tiles * kbt)
+        d = mm.DealtKBlocks(m, n, k, tm, tn, grid)
+        assert len(d.seg_off) == tiles + 1
+        pieces = 0
+        for t in range(tiles):
+            b = d.seg_bounds[d.seg_off[t]:d.seg_off[t + 1]]
+            assert b[0] == 0 and b[-1] == kbt and (np.diff(b) > 0).all()
+            pieces += len(b) - 1
+        # a run of q or q+1 pairs starts a new piece wherever it starts inside a tile, and every tile starts one
+        q, r = divmod(tiles * kbt, grid)
+        starts = {w * q + min(w, r) for w in range(grid)}
+        assert pieces == len(starts | {t * kbt for t in range(tiles)})
+    cpu, expected, _ = golden_gemm
+    m, k = cpu[0].shape
+    n = cpu[1].shape[0]
+    idx = np.stack(np.meshgrid(np.arange(m), np.arange(n), indexing="ij"), -1).reshape(-1, 2)
+    for (tm, tn, grid) in ((16, 16, 4), (16, 32, 2), (64, 128, 2), (16, 16, 3)):
+        cuts = mm.DealtKBlocks(m, n, k, tm, tn, min(grid, -(-m // tm) * -(-n // tn) * (k // 128)))
+        got, _ = mm.model_kernel_at(cpu, idx, cuts)
+        assert torch.equal(got.view(torch.int16), expected.reshape(-1).view(torch.int16)), (tm, tn, grid)
+    # and where the operands are not exact, the cuts show: two pieces summed are not always one chain of fma's
+    rng = torch.Generator().manual_seed(5)
+    from importlib import import_module
+    pkg = import_module("amd-developer-challenge-2025_amd")
+    cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0], m=64, n=64, k=1024)
+    idx = np.stack(np.meshgrid(np.arange(64), np.arange(64), indexing="ij"), -1).reshape(-1, 2)
+    whole, _ = mm.model_kernel_at(cpu, idx, 1)
+    cut, _ = mm.model_kernel_at(cpu, idx, mm.DealtKBlocks(64, 64, 1024, 64, 64, 4))
+    plane, _ = mm.model_kernel_at(cpu, idx, 4)
+    _, whole32 = mm.model_kernel_at(cpu, idx, 1)
+    _, cut32 = mm.model_kernel_at(cpu, idx, mm.DealtKBlocks(64, 64, 1024, 64, 64, 4))
+    _, plane32 = mm.model_kernel_at(cpu, idx, 4)
+    assert (whole32 != cut32).any()                          # four pieces of two K blocks each, not one chain
+    # own piece first, then the others in ascending K: the same four partial sums as a K split of 4, another order
+    assert (cut32 != plane32).any() and torch.allclose(cut32, plane32, rtol=1e-5, atol=1e-3)
