@@ -304,9 +304,9 @@ void gemm_tr_kernel(const GemmArgs p) {
         if (MODE == 3) {
             // K blocks, not tiles, are dealt to the workgroups: the (tile, K block) pairs of the whole product
             // form one sequence - tiles in the band order of the dense walk, K ascending inside a tile - and
-            // workgroup v takes the run of total/G pairs (the first total%G runs hold one more), G <= total.  A run covers the end of one tile,
-            // whole tiles, and the beginning of another; the workgroup walks its tiles from the last to the
-            // first.  A segment that ends before its tile's last K block is stored as an fp32 partial tile in
+            // workgroup v takes a run of total/G pairs (the first total%G runs hold one more), G <= total.  A run
+            // covers the end of one tile, whole tiles, and the beginning of another; the workgroup walks its tiles
+            // from the last to the first.  A segment that ends before its tile's last K block is stored as an fp32 partial tile in
             // the workgroup's slot of the workspace (only the first segment a workgroup works on can be one);
             // the segment that holds the tile's last K block belongs to the tile's owner, who adds the
             // partial tiles of the workgroups before it in ascending order of K, then its own accumulators,
