@@ -96,33 +96,41 @@ bool skinny_shape(int m, int n, int k) { return m <= 64 && (double)n * (double)k
 void choose_tiled(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may_split = true) {
     if (num_cus <= 0) num_cus = 256;
     int kbt = k / KBLK;
-    // The tile shape and K split that finish soonest under a cost model in microseconds.  Per variant
-    // and number r of workgroups resident on a CU: the time in which all r advance one K block, and the
-    // fixed time of a round (prologue, output, drain).  Workgroups are dealt in rounds of (CUs x the most
-    // that fit a CU); a last partial round runs with fewer per CU.  A K split adds the fp32 partial
-    // planes (written and read back, mostly through the 256 MB cache) and the reduce launch.  The
-    // constants are a least-squares fit (of the logarithms) of this model to the measured time of every
+    // The tile shape and K split that finish soonest under a cost model in microseconds.  A workgroup advances one
+    // K block in max(t_alone x f(r), t_power x w / CUs): t_alone is the tile's time per block at the full clock
+    // (f(r) = 1, 1.30, 1.71 with r = 1, 2, 3 workgroups sharing a CU), t_power what the board's power limit allows
+    // when every CU runs one such workgroup - with w workgroups running together the limit is shared by w, so fewer
+    // busy CUs clock higher until the full clock is reached.  A round of workgroups (CUs x the most that fit a CU; a
+    // last partial round with fewer) costs a fixed time for the first copies' latency, the output and the drain.  A
+    // K split adds the fp32 partial planes (written and read back, mostly through the 256 MB cache) and the reduce
+    // launch.  The constants are a least-squares fit (of logarithms) of this model to the measured time of every
     // (tile, split) pair on 38 shapes on MI355X - the 18 of the upstream benchmark and 20 others, M 96 .. 16384,
-    // N 1024 .. 28672, K 1024 .. 14336 - (rms error 14 %; picking by the model costs 2.7 % against picking the
-    // measured best, geometric mean over the shapes, worst shape +17 %).
-    struct Cand { int variant; int rmax; double t_block[3], t_fixed[3]; };
+    // N 1024 .. 28672, K 1024 .. 14336 - (rms error 10 %; picking by the model costs 1.2 % against picking the
+    // measured best, geometric mean over the shapes, worst shape +13 %).
+    struct Cand { int variant; int rmax; double t_alone, t_power, t_fixed; };
     const Cand cands[7] = {
-        {FP8BS_VARIANT_T256x256, 1, {1.227, 0, 0}, {7.15, 0, 0}},
-        {FP8BS_VARIANT_T256x192, 1, {1.058, 0, 0}, {5.84, 0, 0}},
-        {FP8BS_VARIANT_T192x192S3, 1, {0.948, 0, 0}, {4.50, 0, 0}},
-        {FP8BS_VARIANT_T256x128S3, 1, {0.845, 0, 0}, {3.71, 0, 0}},
-        {FP8BS_VARIANT_T128x128, 2, {0.806, 1.177, 0}, {3.07, 2.53, 0}},
-        {FP8BS_VARIANT_T64x128, 3, {0.653, 0.800, 1.396}, {1.97, 2.90, 1.09}},
+        {FP8BS_VARIANT_T256x256, 1, 1.181, 1.462, 6.75},
+        {FP8BS_VARIANT_T256x192, 1, 1.011, 1.163, 5.51},
+        {FP8BS_VARIANT_T192x192S3, 1, 0.881, 1.059, 4.11},
+        {FP8BS_VARIANT_T256x128S3, 1, 0.783, 0.906, 3.70},
+        {FP8BS_VARIANT_T128x128, 2, 0.797, 0.570, 2.86},
+        {FP8BS_VARIANT_T64x128, 3, 0.645, 0.400, 1.91},
         // the 64x256 three-stage tile: many small tiles and a deep copy ring; what shapes of a few hundred rows, or
         // with few K blocks per tile, finish soonest on (1536 x 1536 x 4096: 21.4 us against 25.0 with the best of the others)
-        {FP8BS_VARIANT_T64x256S3, 1, {0.645, 0, 0}, {1.81, 0, 0}},
+        {FP8BS_VARIANT_T64x256S3, 1, 0.576, 0.618, 2.03},
     };
+    const double shared[3] = {1.0, 1.30, 1.71};
     const int splits[6] = {1, 2, 3, 4, 6, 8};
     int best_variant = 0, best_split = 1; double best_cost = 0;
     for (const Cand& c : cands) {
         VariantInfo vi{};
         variant_info(c.variant, &vi);
         const long tiles = cdiv(m, vi.bm) * cdiv(n, vi.bn);
+        auto t_block = [&](long w) {          // w workgroups running together
+            const long r = cdiv(w, num_cus) < c.rmax ? cdiv(w, num_cus) : c.rmax;
+            const double alone = c.t_alone * shared[r - 1], power = c.t_power * (double)w / (double)num_cus;
+            return alone > power ? alone : power;
+        };
         for (int s : splits) {
             // keep at least 4 K blocks per workgroup - 8 with the 64x256 tile, whose short blocks leave a workgroup's
             // first copies and its partial plane as most of its time (1024 x 512 x 7168: split 8 20.9 us, split 4 18.6)
@@ -130,12 +138,9 @@ void choose_tiled(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may_
             const long wgs = tiles * s, per_round = (long)num_cus * c.rmax;
             const long full = wgs / per_round, rem = wgs % per_round;
             const double kb = (double)cdiv(kbt, s);
-            double cost = (double)full * (c.t_fixed[c.rmax - 1] + kb * c.t_block[c.rmax - 1]);
-            if (rem) {
-                const long r = cdiv(rem, num_cus);
-                cost += c.t_fixed[r - 1] + kb * c.t_block[r - 1];
-            }
-            if (s > 1) cost += 3.65 + 0.043 * s + 1.14e-6 * s * (double)m * (double)n;
+            double cost = (double)full * (c.t_fixed + kb * t_block(per_round));
+            if (rem) cost += c.t_fixed + kb * t_block(rem);
+            if (s > 1) cost += 4.85 + 1.10e-6 * s * (double)m * (double)n;
             if (best_variant == 0 || cost < best_cost) { best_variant = c.variant; best_split = s; best_cost = cost; }
         }
     }

@@ -178,6 +178,8 @@ def test_seeded_random_shapes_through_the_planner(pkg, oracle, dev):
             m = int(rng.choice([4, 8, 12, 16])) * int(rng.integers(1, 60)) if i % 3 else 4 * int(rng.integers(1, 40))
             n = 8 * int(rng.integers(1, 140))
         k = 128 * int(rng.integers(1, 13))
+        if i % 5 == 2:
+            k = 128 * int(rng.integers(32, 57))                   # long K against few tiles: the planner splits K
         if i % 2:
             m -= int(rng.integers(1, 4))                          # half of the shapes off the 4-row grid
             m = max(m, 1)

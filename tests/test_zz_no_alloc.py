@@ -50,7 +50,7 @@ def test_without_a_split_and_beyond_the_limit(pkg, dev):
     plan, want, got = _call_both(pkg, dev, pkg.inputs.CONFIGS[0], 256, 512, 1024)          # no K split planned: the array is not touched
     assert plan.split_k == 1 and torch.equal(got.view(torch.int16), want.view(torch.int16))
     # a shape whose planned K split needs more partial-plane bytes than the array holds is refused, nothing is launched
-    m, n, k = 2048, 2048, 16384
+    m, n, k = 2048, 2048, 32768
     plan = pkg.plan(m, n, k)
     assert plan.split_k > 1 and plan.workspace_bytes > SCRATCH_LIMIT
     a = torch.zeros(k, m, dtype=torch.uint8, device=dev)
