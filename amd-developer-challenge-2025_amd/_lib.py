@@ -27,8 +27,12 @@ class Plan(ctypes.Structure):
         ("variant", ctypes.c_int32), ("tile_m", ctypes.c_int32), ("tile_n", ctypes.c_int32),
         ("split_k", ctypes.c_int32), ("grid_x", ctypes.c_int32), ("grid_y", ctypes.c_int32),
         ("grid_z", ctypes.c_int32), ("block_threads", ctypes.c_int32), ("lds_bytes", ctypes.c_int32),
-        ("stream_k", ctypes.c_int32), ("workspace_bytes", ctypes.c_uint64),
+        ("stream_k", ctypes.c_int32), ("sum_in_kernel", ctypes.c_int32), ("reserved", ctypes.c_int32),
+        ("workspace_bytes", ctypes.c_uint64),
     ]
+
+
+SPLIT_SUM_IN_KERNEL = 1 << 30        # FP8BS_SPLIT_SUM_IN_KERNEL
 
 
 _lib = None

@@ -58,8 +58,22 @@ int streamk_grid(int variant, int m, int n, int k, int num_cus) {
     return (int)(g < fp8bs::StreamK::MAX_GRID ? g : fp8bs::StreamK::MAX_GRID);
 }
 
-// Fill a plan for a given variant and split count.
-void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out, int stream_k = 0) {
+bool is_streaming_variant(int v) { return v == FP8BS_VARIANT_SKINNY64x144 || v == FP8BS_VARIANT_SKINNY64x256 || v == FP8BS_VARIANT_SKINNY64x288; }
+
+// The fp32 partial planes of a K split followed by the reduce kernel.
+uint64_t planes_bytes(int m, int n, int split_k) { return split_k > 1 ? (uint64_t)split_k * (uint64_t)m * (uint64_t)n * 4u : 0u; }
+
+// Can the partial tiles of a K split of this tile shape be summed in the kernel that writes them (one counter per
+// tile in the head of the workspace, the partition count in the counter's low 16 bits)?
+bool can_sum_in_kernel(int m, int n, int variant, int split_k) {
+    VariantInfo vi{};
+    if (variant == FP8BS_VARIANT_GENERIC || is_streaming_variant(variant) || !variant_info(variant, &vi)) return false;
+    return split_k >= 2 && split_k <= 255 && cdiv(m, vi.bm) * cdiv(n, vi.bn) <= fp8bs::StreamK::MAX_GRID;
+}
+
+// Fill a plan for a given variant and split count.  in_kernel: the split's partial tiles are summed by the last
+// workgroup to finish each tile (where the shape allows it, see above; else the reduce kernel follows).
+void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out, int stream_k = 0, bool in_kernel = false) {
     VariantInfo vi{};
     variant_info(variant, &vi);
     int kbt = k / KBLK;
@@ -74,13 +88,17 @@ void fill_plan(int m, int n, int k, int variant, int split_k, fp8bs_plan_t* out,
     out->block_threads = vi.threads;
     out->lds_bytes = fp8bs::variant_lds_bytes(variant);
     out->stream_k = stream_k > 0 ? stream_k : 0;
+    out->sum_in_kernel = in_kernel && stream_k <= 0 && can_sum_in_kernel(m, n, variant, split_k) ? 1 : 0;
+    out->reserved = 0;
     if (variant == FP8BS_VARIANT_GENERIC) {
         out->grid_x = (int)cdiv(n, 16); out->grid_y = (int)cdiv(m, 16); out->grid_z = 1;
     } else {
         out->grid_x = stream_k > 0 ? stream_k : (int)(cdiv(m, vi.bm) * cdiv(n, vi.bn) * split_k); out->grid_y = 1; out->grid_z = 1;
     }
-    out->workspace_bytes = stream_k > 0 ? (uint64_t)fp8bs::StreamK::bytes(stream_k, vi.bm, vi.bn)
-                                        : (split_k > 1 ? (uint64_t)split_k * (uint64_t)m * (uint64_t)n * 4u : 0u);
+    if (stream_k > 0) out->workspace_bytes = (uint64_t)fp8bs::StreamK::bytes(stream_k, vi.bm, vi.bn);
+    else if (out->sum_in_kernel)   // the counters, then one fp32 tile per (tile, K partition)
+        out->workspace_bytes = (uint64_t)fp8bs::StreamK::SLOTS_OFF + (uint64_t)(cdiv(m, vi.bm) * cdiv(n, vi.bn)) * (uint64_t)split_k * (uint64_t)vi.bm * (uint64_t)vi.bn * 4u;
+    else out->workspace_bytes = planes_bytes(m, n, split_k);
 }
 
 // Rows of c (n bf16) that keep 16-byte stores aligned: what the streaming kernels need (forced variants only;
@@ -121,7 +139,7 @@ void choose_tiled(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may_
     };
     const double shared[3] = {1.0, 1.30, 1.71};
     const int splits[6] = {1, 2, 3, 4, 6, 8};
-    int best_variant = 0, best_split = 1; double best_cost = 0;
+    int best_variant = 0, best_split = 1; double best_cost = 0; bool best_fused = false;
     for (const Cand& c : cands) {
         VariantInfo vi{};
         variant_info(c.variant, &vi);
@@ -140,11 +158,19 @@ void choose_tiled(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may_
             const double kb = (double)cdiv(kbt, s);
             double cost = (double)full * (c.t_fixed + kb * t_block(per_round));
             if (rem) cost += c.t_fixed + kb * t_block(rem);
-            if (s > 1) cost += 4.85 + 1.10e-6 * s * (double)m * (double)n;
-            if (best_variant == 0 || cost < best_cost) { best_variant = c.variant; best_split = s; best_cost = cost; }
+            // the planes and the reduce launch; or, with two or three partitions, the sum in the kernel: no second
+            // launch and no pass over whole planes, but the last workgroup of a tile reads s - 1 partial tiles alone
+            // (measured on the same 38 shapes: two partitions 1-50 us faster than with the reduce launch, median 4.7;
+            // three: median 2.3 faster; four and more: the serial sums cost more than the launch)
+            const double planes = 4.85 + 1.10e-6 * s * (double)m * (double)n;
+            const double in_kernel = 3.77 + 0.752e-6 * s * (double)m * (double)n
+                                     + 5.90 * (s - 1) * (vi.bm * vi.bn * 4e-6) * (double)cdiv(wgs, num_cus);
+            const bool fuse = (s == 2 || s == 3) && can_sum_in_kernel(m, n, c.variant, s) && in_kernel < planes;
+            if (s > 1) cost += fuse ? in_kernel : planes;
+            if (best_variant == 0 || cost < best_cost) { best_variant = c.variant; best_split = s; best_cost = cost; best_fused = fuse; }
         }
     }
-    fill_plan(m, n, k, best_variant, best_split, out);
+    fill_plan(m, n, k, best_variant, best_split, out, 0, best_fused);
 }
 
 // Skinny shapes: the 64 x 256 tile with three LDS stages (two K blocks of b, 64 KB, in flight per workgroup) and
@@ -169,9 +195,12 @@ void choose_skinny(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may
         if (t_block < 1.05) t_block = 1.05;
         double cost = (double)cdiv(wgs, num_cus) * (2.0 + (double)cdiv(kbt, s) * t_block);
         if (s > 1) cost += 4.0 + 0.24 * s + 1.19e-6 * s * (double)m * (double)n;
+        // two or three partitions are summed in the kernel (64 x 18432 x 7168, b from HBM: 33.5 us against 34.4 with
+        // three, 37.4 against 38.6 with two; with four 52.8 against 49.6)
+        if (s == 2 || s == 3) cost -= 0.8;
         if (s == 1 || cost < best) { best = cost; best_s = s; }
     }
-    fill_plan(m, n, k, FP8BS_VARIANT_T64x256S3, best_s, out);
+    fill_plan(m, n, k, FP8BS_VARIANT_T64x256S3, best_s, out, 0, best_s == 2 || best_s == 3);
 }
 
 // Shape-family rule.  A few rows against a large b -> the 64 x 256 three-stage tile.  Everything else -> the
@@ -210,7 +239,6 @@ int streamk_spin_limit() {
     return limit;
 }
 
-bool is_streaming_variant(int v) { return v == FP8BS_VARIANT_SKINNY64x144 || v == FP8BS_VARIANT_SKINNY64x256 || v == FP8BS_VARIANT_SKINNY64x288; }
 
 int check_common(const void* a, const void* b, const float* as, const float* bs, void* c, int m, int n, int k) {
     if (m < 0 || n < 0 || k < 0 || (k % KBLK) != 0) return FP8BS_ERR_BAD_SHAPE;
@@ -313,10 +341,15 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
     const int cus = fp8bs::device_cus();
     if (variant == FP8BS_VARIANT_AUTO) {
         choose(m, n, k, cus, &plan);
-        if (split_k > 0) fill_plan(m, n, k, plan.variant, split_k, &plan);
+        if (split_k > 0) fill_plan(m, n, k, plan.variant, split_k & ~FP8BS_SPLIT_SUM_IN_KERNEL, &plan, 0, (split_k & FP8BS_SPLIT_SUM_IN_KERNEL) != 0);
         else if (split_k < 0) fill_plan(m, n, k, plan.variant, 1, &plan, streamk_grid(plan.variant, m, n, k, cus));
         // the plan needs a workspace the caller did not bring: the best plan that needs none
-        else if (plan.workspace_bytes > 0 && (!ws || ws_bytes < plan.workspace_bytes)) choose(m, n, k, cus, &plan, false);
+        else if (plan.workspace_bytes > 0 && (!ws || ws_bytes < plan.workspace_bytes)) {
+            // too small for the partial tiles of a sum in the kernel but not for the planes (tiles that overhang
+            // the matrix): the same split with the reduce kernel
+            if (plan.sum_in_kernel && ws && ws_bytes >= planes_bytes(m, n, plan.split_k)) fill_plan(m, n, k, plan.variant, plan.split_k, &plan);
+            else choose(m, n, k, cus, &plan, false);
+        }
     } else {
         VariantInfo vi{};
         if (!variant_info(variant, &vi)) return FP8BS_ERR_BAD_VARIANT;
@@ -326,7 +359,9 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
             if (is_streaming_variant(variant) || variant == FP8BS_VARIANT_GENERIC) return FP8BS_ERR_BAD_VARIANT;   // K blocks are dealt by the tiled kernel only
             fill_plan(m, n, k, variant, 1, &plan, streamk_grid(variant, m, n, k, cus));
         } else {
-            fill_plan(m, n, k, variant, split_k > 0 ? split_k : 1, &plan);
+            const bool in_kernel = split_k > 0 && (split_k & FP8BS_SPLIT_SUM_IN_KERNEL) != 0;
+            if (in_kernel && (is_streaming_variant(variant) || variant == FP8BS_VARIANT_GENERIC)) return FP8BS_ERR_BAD_VARIANT;   // the tiled kernel only
+            fill_plan(m, n, k, variant, split_k > 0 ? (split_k & ~FP8BS_SPLIT_SUM_IN_KERNEL) : 1, &plan, 0, in_kernel);
         }
     }
     if (plan.workspace_bytes > 0 && (!ws || ws_bytes < plan.workspace_bytes)) return FP8BS_ERR_WORKSPACE;
@@ -340,7 +375,10 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
     g.band_h = 4;
     g.num_experts = 0;
     int mode = plan.split_k > 1 ? 1 : 0;
-    if (plan.stream_k > 0) {
+    if (plan.sum_in_kernel && plan.split_k > 1) {
+        mode = 4;
+        g.sk_nonce = next_nonce();
+    } else if (plan.stream_k > 0) {
         mode = 3;
         g.sk_grid = plan.stream_k;
         g.sk_nonce = next_nonce();
@@ -367,13 +405,15 @@ int fp8bs_gemm_noalloc(const void* a, const void* b, const float* a_scale, const
     fp8bs_plan_t plan{};
     if (k > 0) {
         choose(m, n, k, fp8bs::device_cus(), &plan);
-        if (plan.workspace_bytes > (uint64_t)FP8BS_NOALLOC_SCRATCH_BYTES) return FP8BS_ERR_SCRATCH_LIMIT;
+        uint64_t need = plan.workspace_bytes;
+        if (plan.sum_in_kernel && planes_bytes(m, n, plan.split_k) < need) need = planes_bytes(m, n, plan.split_k);   // fp8bs_gemm_ex falls back to the planes
+        if (need > (uint64_t)FP8BS_NOALLOC_SCRATCH_BYTES) return FP8BS_ERR_SCRATCH_LIMIT;
     }
     void* ws = nullptr;
     st = scratch_address(&ws, (hipStream_t)stream);
     if (st != FP8BS_OK) return st;
-    // Every partial element that the reduction reads is written by this call's main kernel first, so
-    // nothing in the array has to start at zero.
+    // Every partial element that the sum reads is written by this call first, and a tile's counter in the head
+    // of the array counts only arrivals that carry this call's tag, so nothing in the array has to start at zero.
     return fp8bs_gemm_ex(a, b, a_scale, b_scale, c, ws, (size_t)FP8BS_NOALLOC_SCRATCH_BYTES, m, n, k, FP8BS_VARIANT_AUTO, 0, stream);
 }
 

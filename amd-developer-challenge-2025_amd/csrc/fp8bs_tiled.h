@@ -103,6 +103,8 @@ __device__ __forceinline__ void band_tile(int v, int tiles_m, int tiles_n, int g
 //   MODE 0  : dense, bf16 output
 //   MODE 1  : dense split-K, fp32 partial planes to the workspace
 //   MODE 2  : grouped (row_offsets), bf16 output
+//   MODE 3  : dense, K blocks instead of tiles dealt to the workgroups, partial tiles through the workspace, bf16 output
+//   MODE 4  : dense split-K, partial tiles to the workspace, summed by the last workgroup to finish a tile, bf16 output
 // LDS: 2 stages, each [128 k][BM] bytes of A then [128 k][BN] bytes of B, 16-byte chunks XOR-swizzled
 // so that the 16 k rows touched by half a wave in one transposing read fall on 16 different 16-byte
 // bank groups, then the k block's a_scale row and b_scale values.
@@ -216,8 +218,19 @@ __device__ __forceinline__ float silu_mul(float gate, float up) {
 // TAILS: lda is not a multiple of four or n not a multiple of eight; the kernel then repairs the last
 // bytes of a and b in LDS (one more barrier per tile) and stores a row's last, partial 16-byte chunk of c
 // in pieces, see below.
+// Waves per SIMD when as many workgroups as LDS and thread count allow share a CU.  The modes that exchange partial
+// tiles must keep their registers within that (their sums would otherwise take registers the K loop does not need
+// and halve the number of workgroups per CU); the other modes fit without being told.
+template <int BM, int BN, int WM, int WN, int MODE, int NSTAGE>
+constexpr int waves_per_simd() {
+    using C = TileCfg<BM, BN, WM, WN, MODE, NSTAGE>;
+    const int by_lds = 163840 / C::LDS_BYTES, by_threads = 2048 / C::NTHREADS;
+    const int w = C::NWAVES * (by_lds < by_threads ? by_lds : by_threads) / 4;
+    return MODE >= 3 && w > 1 ? w : 1;
+}
+
 template <int BM, int BN, int WM, int WN, int MODE, int EPI = 0, int NSTAGE = 2, bool TAILS = false>
-__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64)
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) __attribute__((amdgpu_waves_per_eu(waves_per_simd<BM, BN, WM, WN, MODE, NSTAGE>())))
 void gemm_tr_kernel(const GemmArgs p) {
     using C = TileCfg<BM, BN, WM, WN, MODE, NSTAGE>;
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
@@ -415,6 +428,7 @@ void gemm_tr_kernel(const GemmArgs p) {
             t.split_z = v / per_split;
             int tm, tn;
             band_tile(v - t.split_z * per_split, tiles_m, tiles_n, p.band_h, tm, tn);
+            if (MODE == 4) t.sk_first = v - t.split_z * per_split;        // the tile's number: its counter and its slots
             t.m0 = tm * BM; t.n0 = tn * BN;
             const int kbt = p.k / KBLK;
             t.kb_begin = t.split_z * p.kb_per_split;
@@ -908,6 +922,134 @@ void gemm_tr_kernel(const GemmArgs p) {
                 }
             }
         }
+    } else if constexpr (MODE == 4) {
+        // K split in one launch, nobody waits: every workgroup leaves its partial tile in the slot
+        // (tile, K partition) and then counts itself in at the tile's counter; the one that finds all others
+        // counted in before it adds the partial tiles in ascending order of K - ((P0 + P1) + P2) + ..., its own
+        // from the registers, the order of the separate reduce kernel - and writes the bf16 tile.  The counter
+        // carries the call's tag in its upper 48 bits, so whatever an earlier use of the workspace left there
+        // counts as zero; the last workgroup puts it back to zero for a replay of the same launch.
+        constexpr uint32_t SLOT_BYTES = (uint32_t)BM * (uint32_t)BN * 4u;
+        constexpr int NG = C::MT * C::NT;
+        constexpr int AUX_AGENT = 16;                                           // sc1
+        __shared__ int last_in;
+        unsigned char* const ws_base = (unsigned char*)p.ws;
+        unsigned long long* const counters = (unsigned long long*)(ws_base + StreamK::FLAGS_OFF);
+        unsigned char* const tile_slots = ws_base + StreamK::SLOTS_OFF + (size_t)sk_first * (size_t)p.split_k * SLOT_BYTES;
+        const uint32_t voff = (uint32_t)(wave * NG) * 1024u + (uint32_t)lane * 16u;
+        // (the counter is read ahead of the stores: the value only seeds the exchange below, which finds out if it is stale)
+        unsigned long long seen = 0;
+        if (tid == 0) seen = __hip_atomic_load(&counters[sk_first], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (wave_active) {
+            __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(tile_slots + (size_t)split_z * SLOT_BYTES), 0, SLOT_BYTES, 0x00020000);
+#pragma unroll
+            for (int t = 0; t < C::MT; t++)
+#pragma unroll
+                for (int u = 0; u < C::NT; u++)
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, acc[t][u]), rs, voff + (uint32_t)(t * C::NT + u) * 1024u, 0, AUX_AGENT);
+        }
+        wait_vmcnt<0>();                                    // acknowledged from the agent's point of coherence
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned long long tag = (p.sk_nonce | 0x10000ull) & ~0xFFFFull;       // never zero
+            unsigned long long count;
+            for (;;) {
+                count = (seen & ~0xFFFFull) == tag ? (seen & 0xFFFFull) : 0ull;
+                if (__hip_atomic_compare_exchange_strong(&counters[sk_first], &seen, tag | (count + 1), __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
+            }
+            const int last = (int)(count + 1) == p.split_k;
+            if (last) __hip_atomic_store(&counters[sk_first], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_in = last;
+        }
+        __syncthreads();
+        store_output = __builtin_amdgcn_readfirstlane(last_in) != 0;
+        if (store_output && wave_active) {
+            __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)tile_slots, 0, (uint32_t)p.split_k * SLOT_BYTES, 0x00020000);
+            // S partitions known at compile time: the loads of all other partitions' pieces of a batch are in flight
+            // together (up to 16 of 16 bytes per lane); S = 0: any number, one partition at a time
+            [[maybe_unused]] auto sum_planes = [&]<int S>() {
+                constexpr int WANT = S > 1 ? (16 / (S - 1) > 0 ? 16 / (S - 1) : 1) : 4;
+                constexpr int BATCH = WANT >= NG ? NG : (WANT >= 4 && NG % 4 == 0 ? 4 : (WANT >= 3 && NG % 3 == 0 ? 3 : (WANT >= 2 && NG % 2 == 0 ? 2 : 1)));
+                const int nz = S > 0 ? S : p.split_k;
+#pragma unroll
+                for (int base = 0; base < NG; base += BATCH) {
+                    if constexpr (S > 0) {
+                        v4f part[S - 1][BATCH];                              // the other partitions, ascending
+#pragma unroll
+                        for (int j = 0; j < S - 1; j++) {
+                            const uint32_t soff = (uint32_t)(j + (j >= split_z ? 1 : 0)) * SLOT_BYTES;
+#pragma unroll
+                            for (int i = 0; i < BATCH; i++)
+                                part[j][i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff + (uint32_t)(base + i) * 1024u, AUX_AGENT));
+                        }
+#pragma unroll
+                        for (int i = 0; i < BATCH; i++) {
+                            v4f& own = acc[(base + i) / C::NT][(base + i) % C::NT];
+                            v4f sum = part[0][i];
+                            if (split_z == 0) sum = own + sum;                  // (the same bits as sum + own)
+#pragma unroll
+                            for (int j = 1; j < S - 1; j++) {
+                                if (j == split_z) sum += own;
+                                sum += part[j][i];
+                            }
+                            if (split_z == S - 1) sum += own;
+                            own = sum;
+                        }
+                    } else {
+                        v4f sum[BATCH];
+                        for (int z = 0; z < nz; z++) {
+                            v4f part[BATCH];
+                            if (z == split_z) {
+#pragma unroll
+                                for (int i = 0; i < BATCH; i++) part[i] = acc[(base + i) / C::NT][(base + i) % C::NT];
+                            } else {
+#pragma unroll
+                                for (int i = 0; i < BATCH; i++)
+                                    part[i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs, voff, (uint32_t)z * SLOT_BYTES + (uint32_t)(base + i) * 1024u, AUX_AGENT));
+                            }
+#pragma unroll
+                            for (int i = 0; i < BATCH; i++) sum[i] = z == 0 ? part[i] : sum[i] + part[i];
+                        }
+#pragma unroll
+                        for (int i = 0; i < BATCH; i++) acc[(base + i) / C::NT][(base + i) % C::NT] = sum[i];
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            };
+            if constexpr (NG > 16) {
+                // 72 to 128 accumulator registers leave room for one partition's batch of three or four
+                constexpr int GB = NG % 4 == 0 ? 4 : (NG % 3 == 0 ? 3 : (NG % 2 == 0 ? 2 : 1));
+#pragma unroll
+                for (int base = 0; base < NG; base += GB) {
+                    v4f sum[GB];
+                    for (int z = 0; z < p.split_k; z++) {
+                        v4f part[GB];
+                        if (z == split_z) {
+#pragma unroll
+                            for (int i = 0; i < GB; i++) part[i] = acc[(base + i) / C::NT][(base + i) % C::NT];
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < GB; i++)
+                                part[i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs, voff, (uint32_t)z * SLOT_BYTES + (uint32_t)(base + i) * 1024u, AUX_AGENT));
+                        }
+#pragma unroll
+                        for (int i = 0; i < GB; i++) sum[i] = z == 0 ? part[i] : sum[i] + part[i];
+                    }
+#pragma unroll
+                    for (int i = 0; i < GB; i++) acc[(base + i) / C::NT][(base + i) % C::NT] = sum[i];
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+                switch (p.split_k) {
+                    case 2: sum_planes.template operator()<2>(); break;
+                    case 3: sum_planes.template operator()<3>(); break;
+                    case 4: sum_planes.template operator()<4>(); break;
+                    case 5: sum_planes.template operator()<5>(); break;
+                    case 6: sum_planes.template operator()<6>(); break;
+                    default: sum_planes.template operator()<0>(); break;
+                }
+            }
+        }
     }
 
     // ---- epilogue (a wave without valid rows has nothing to store; no barrier in here) -----------
@@ -1113,6 +1255,12 @@ static inline hipError_t launch_shape(const GemmArgs& a, int mode, hipStream_t s
         return launch_tr<BM, BN, WM, WN, 3, 0, NSTAGE>(a, dim3((unsigned)a.sk_grid), stream);
     }
     const dim3 grid((unsigned)(total < resident ? total : resident));
+    if (mode == 4) {
+        // K split summed by the last workgroup of every tile: one counter per tile in the workspace's head
+        const long tiles = total / a.split_k;
+        if (a.epi != 0 || a.split_k < 2 || a.split_k > 0xFFFF || tiles > StreamK::MAX_GRID || (long)a.split_k * BM * BN * 4 >= (1L << 32)) return hipErrorInvalidValue;
+        return launch_tr<BM, BN, WM, WN, 4, 0, NSTAGE>(a, grid, stream);
+    }
     if (a.epi != 0) {
         // the fused silu-mul epilogue exists for the 256x256 tile, dense or grouped, without K split
         if constexpr (WITH_EPI) {

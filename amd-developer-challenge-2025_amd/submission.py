@@ -133,8 +133,9 @@ def workspace_bytes(m: int, n: int, k: int) -> int:
 def custom_kernel(data, variant: int = 0, split_k: int = 0):
     """Block-scale fp8 gemm: fills and returns ``c`` (see module docstring for the layouts).
 
-    ``variant``/``split_k`` force a kernel variant (FP8BS_VARIANT_*) and a K split for testing;
-    the defaults let the library's planner decide.
+    ``variant``/``split_k`` force a kernel variant (FP8BS_VARIANT_*) and a K split for testing
+    (``split_k | SPLIT_SUM_IN_KERNEL``: the partitions summed in the one kernel; ``split_k < 0``: K blocks
+    dealt to the workgroups); the defaults let the library's planner decide.
     """
     a, b, a_scale, b_scale, c = data
     gemm_ex = _gemm_ex or _bind()[0]
@@ -177,6 +178,9 @@ def custom_kernel(data, variant: int = 0, split_k: int = 0):
         # a forced K split's planes; K blocks dealt to the workgroups (split_k < 0): a header and one fp32 tile per
         # workgroup, at most 64 MiB for every tile shape on 256 CUs
         need = split_k * m * n * 4 if split_k > 1 else ((64 << 20) + 16384 if split_k < 0 else 0)
+        if split_k > 0 and split_k & _lib.SPLIT_SUM_IN_KERNEL:
+            # summed in the kernel: a header and split_k fp32 tiles per tile (the largest tile is 256 x 256)
+            need = 16384 + (split_k & ~_lib.SPLIT_SUM_IN_KERNEL) * (m + 255) * (n + 255) * 4
     # kernels are launched on the device the pointers live on: the library uses the current device
     with torch.cuda.device(a.device):
         stream = _stream_ptr(a.device)

@@ -77,8 +77,15 @@ typedef struct fp8bs_plan_t {
     int32_t lds_bytes;
     int32_t stream_k;       /* > 0: K blocks, not tiles, are dealt to this many workgroups (one launch;
                                partial tiles meet in the workspace); split_k is 1 then           */
+    int32_t sum_in_kernel;  /* 1 (with split_k > 1): one launch - the workgroups of a tile's K partitions leave fp32
+                               partial tiles in the workspace and the last one to finish adds them in ascending K and
+                               writes c; 0: partial planes and a reduce kernel (two launches)      */
+    int32_t reserved;
     uint64_t workspace_bytes;
 } fp8bs_plan_t;
+
+/* Or'ed into a positive split_k of fp8bs_gemm_ex: sum the K partitions in the kernel (see sum_in_kernel). */
+#define FP8BS_SPLIT_SUM_IN_KERNEL (1 << 30)
 
 /* Library version (major*10000 + minor*100 + patch). */
 int fp8bs_version(void);
@@ -93,7 +100,8 @@ const char* fp8bs_strerror(int status);
  * fp8bs_gemm runs the best plan that needs none (slower, same result up to the summation order). */
 int fp8bs_plan(int m, int n, int k, int num_cus, fp8bs_plan_t* out);
 
-/* Bytes of device workspace fp8bs_gemm needs for this shape (0 when split_k == 1). Replaces the
+/* Bytes of device workspace fp8bs_gemm needs for this shape (0 when split_k == 1; the partial planes, or the
+ * counters and partial tiles of a split summed in the kernel). Replaces the
  * per-call `torch.empty(m*n*4)` of 1-amd-fp8-mm/amd-fp8-mm-submission.py:600: the caller owns and
  * reuses the workspace. */
 size_t fp8bs_workspace_bytes(int m, int n, int k);
@@ -112,8 +120,17 @@ int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* 
 /* Same as fp8bs_gemm with the variant and split-K forced (testing and benchmarking the shape
  * families against each other). variant = FP8BS_VARIANT_AUTO and split_k = 0 reproduce fp8bs_gemm.
  * Workspace requirement for a forced split_k > 1: split_k * m * n * 4 bytes.
- * split_k < 0: the K split in ONE launch - the role of the reference's split kernel plus merge kernel
- * (1-amd-fp8-mm/amd-fp8-mm-submission.py:371-511) without the second launch.  K blocks, not tiles, are dealt to
+ * split_k | FP8BS_SPLIT_SUM_IN_KERNEL: the same K partitions in ONE launch - the role of the reference's split
+ * kernel plus merge kernel (1-amd-fp8-mm/amd-fp8-mm-submission.py:371-511) without the second launch, and what
+ * fp8bs_plan chooses for splits in two or three (sum_in_kernel of the plan).  Every workgroup writes its fp32
+ * partial tile to the workspace and then counts itself in at the tile's counter there; the one that finds all
+ * the others counted in adds the partial tiles in ascending K, its own from its registers - the order of the
+ * reduce kernel, so c holds the same bits as with two launches - and writes c.  Nobody waits for anybody.  The
+ * tiled variants only (else FP8BS_ERR_BAD_VARIANT); with more than 2016 tiles or more than 255 partitions the
+ * call takes the two-launch form.  Workspace: 16384 + tiles * split_k * tile_m * tile_n * 4 bytes
+ * (FP8BS_ERR_WORKSPACE if smaller), contents unspecified on entry (a counter carries the call's own tag, so
+ * whatever an earlier use left there counts as zero), one call at a time per workspace.
+ * split_k < 0: another one-launch form, K BLOCKS instead of tiles dealt to
  * the workgroups (one per place on the chip, G = min(places, tiles * K/128); the tiled variants only, else
  * FP8BS_ERR_BAD_VARIANT); a workgroup whose run of K blocks ends inside a tile leaves an fp32 partial tile in the
  * workspace and raises a flag there, the workgroup that holds the tile's last K block waits for the flags (a
@@ -124,8 +141,8 @@ int fp8bs_gemm(const void* a, const void* b, const float* a_scale, const float* 
  * and the kernel still runs to its end (c is then not valid); nothing else ever writes that word, so a caller
  * that means to read it zeroes it once after allocating.  The environment variable FP8BS_STREAMK_SPIN, read once,
  * sets the polls per flag (default 262144, about a quarter of a second; negative: every wait gives up at once).
- * Measured on MI355X this form is not faster than the planned K split with its reduce launch, so fp8bs_plan
- * never chooses it (stream_k of a plan is 0). */
+ * Measured on MI355X this form is not faster than the planned K split, so fp8bs_plan never chooses it
+ * (stream_k of a plan is 0). */
 int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale,
                   void* c, void* ws, size_t ws_bytes, int m, int n, int k,
                   int variant, int split_k, void* stream);
@@ -133,10 +150,10 @@ int fp8bs_gemm_ex(const void* a, const void* b, const float* a_scale, const floa
 /* fp8bs_gemm for callers that cannot allocate device memory or hand over a workspace: code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference
  * (its split-K path allocates a tensor per call, 1-amd-fp8-mm/amd-fp8-mm-submission.py:600).  Same
- * arguments, plan, kernels and results as fp8bs_gemm, but the fp32 partial planes of a K split live in an
+ * arguments, plan, kernels and results as fp8bs_gemm, but the fp32 partial planes or tiles of a K split live in an
  * array of FP8BS_NOALLOC_SCRATCH_BYTES that is part of the library's device code (every GPU the library
  * runs on holds it until the process ends).  Calls no hipMalloc / hipFree or any allocating routine.
- * A shape whose planned K split needs more partial-plane bytes than that returns FP8BS_ERR_SCRATCH_LIMIT
+ * A shape whose planned K split needs more workspace than that returns FP8BS_ERR_SCRATCH_LIMIT
  * and launches nothing.  All calls on one GPU share the one array: calls that overlap on a GPU (two
  * streams, two threads) race on it; calls on one stream are ordered and safe.  Nothing in the array has to
  * be cleared between calls (every partial element read was written by the same call).

@@ -47,6 +47,16 @@ def test_plan_with_the_devices_cu_count(pkg):
         assert a.stream_k == 0 and a.workspace_bytes == pkg.workspace_bytes(*shape)
 
 
+def _planned_workspace(p, m, n):
+    """What a plan's K split needs: counters and one fp32 tile per (tile, partition) when the partitions are summed in
+    the kernel, whole fp32 planes when a reduce kernel follows."""
+    if p.split_k == 1:
+        return 0
+    if p.sum_in_kernel:
+        return 16384 + -(-m // p.tile_m) * -(-n // p.tile_n) * p.split_k * p.tile_m * p.tile_n * 4
+    return p.split_k * m * n * 4
+
+
 def test_plan_shape_families(pkg):
     p = pkg.plan(4096, 4096, 4096)
     assert p.variant == 2 and (p.tile_m, p.tile_n) == (256, 256) and p.split_k == 1 and p.workspace_bytes == 0
@@ -54,18 +64,19 @@ def test_plan_shape_families(pkg):
     p = pkg.plan(64, 18432, 7168)                       # skinny-M: the 64x256 tile with three stages, 72 tiles x a K split of 3
     assert p.variant == 12 and (p.tile_m, p.tile_n) == (64, 256) and p.split_k == 3 and p.grid_x == 216
     assert p.block_threads == 512 and p.lds_bytes == 3 * (128 * 320 + 1024 + 256)
-    assert p.workspace_bytes == p.split_k * 64 * 18432 * 4 == pkg.workspace_bytes(64, 18432, 7168)
+    assert p.sum_in_kernel == 1                          # three partitions: summed by the last workgroup of each tile, one launch
+    assert p.workspace_bytes == 16384 + 72 * 3 * 64 * 256 * 4 == pkg.workspace_bytes(64, 18432, 7168)
     p = pkg.plan(130, 190, 256)                         # n not a multiple of 8, short K -> a tiled kernel without a K split
     assert p.variant in (2, 3, 4, 9, 10, 11, 12) and p.split_k == 1
     p, q = pkg.plan(1024, 190, 7168), pkg.plan(1024, 192, 7168)   # long K, few tiles: a K split, also with n off the 8-column grid
     assert p.variant == q.variant and p.variant in (2, 3, 4, 9, 10, 11, 12) and p.split_k == q.split_k > 1
-    assert p.workspace_bytes == p.split_k * 1024 * 190 * 4
+    assert p.workspace_bytes == _planned_workspace(p, 1024, 190) and (p.sum_in_kernel == 1) == (p.split_k in (2, 3))
     for m in (130, 4095, 3, 1):                               # any m: the tiled kernels, one launch, nothing extra in the workspace
         p, q = pkg.plan(m, 192, 256), pkg.plan((m + 3) & ~3, 192, 256)
         assert p.variant == q.variant and p.variant not in (1, 6, 7, 8) and p.split_k == q.split_k
-        assert p.workspace_bytes == (p.split_k * m * 192 * 4 if p.split_k > 1 else 0)
+        assert p.workspace_bytes == _planned_workspace(p, m, 192)
     p, q = pkg.plan(3, 18432, 7168), pkg.plan(4, 18432, 7168) # a few rows against a large b: the same skinny plan for any m
-    assert p.variant == q.variant == 12 and p.split_k == q.split_k and p.workspace_bytes == p.split_k * 3 * 18432 * 4
+    assert p.variant == q.variant == 12 and p.split_k == q.split_k and p.workspace_bytes == q.workspace_bytes == _planned_workspace(p, 3, 18432)
     assert pkg.plan(3, 190, 256).variant in (3, 4, 12)
     p = pkg.plan(256, 512, 1024)                        # small: one of the sub-256 tiles, never the scalar kernel
     assert p.variant in (3, 4, 10, 12) and p.split_k >= 1 and p.split_k <= 8
@@ -93,7 +104,8 @@ def test_plan_skinny_rule_and_the_streaming_kernels(pkg):
         if skinny:
             assert p.variant == 12 and p.grid_x == -(-n // 256) * p.split_k, (m, n, k, p.variant)
         assert p.variant not in (1, 6, 7, 8)
-        assert 1 <= p.split_k <= 8 and p.workspace_bytes == (p.split_k * m * n * 4 if p.split_k > 1 else 0)
+        assert 1 <= p.split_k <= 8 and p.workspace_bytes == _planned_workspace(p, m, n)
+        assert p.sum_in_kernel == (1 if p.split_k in (2, 3) else 0)     # two or three partitions are summed in the kernel
     assert pkg.plan(1536, 1536, 4096).variant == 12           # the cost model's pick for a few hundred rows per tile column
     for m in (1, 5, 63):                                      # rows that are not a multiple of four: the same plan
         p, q = pkg.plan(m, 18432, 7168), pkg.plan((m + 3) & ~3, 18432, 7168)

@@ -1,0 +1,174 @@
+"""K split summed in the kernel (fp8bs_gemm_ex with split_k | FP8BS_SPLIT_SUM_IN_KERNEL; what fp8bs_plan picks for
+splits in two or three): one launch, every workgroup leaves its fp32 partial tile in the workspace, the last one to
+finish a tile adds them in ascending K and writes c.
+
+Held to the bar of every other path against the oracle, to the instruction-level model bit for bit, and - because
+the order of the sum is the reduce kernel's - to the bits of the two-launch split.  The reference splits K with a
+second kernel that merges the planes (1-amd-fp8-mm/amd-fp8-mm-submission.py:371-511); this is that work without
+the second launch.
+"""
+import importlib
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 2e-2, 1e-3
+TILED = (2, 3, 4, 9, 10, 11, 12)
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need the GPU box"
+    return torch.device("cuda:0")
+
+
+def _to(data, dev):
+    return tuple(t.to(dev) if isinstance(t, torch.Tensor) else t for t in data)
+
+
+def _bits(t):
+    return t.view(torch.int16)
+
+
+@pytest.mark.parametrize("variant", TILED)
+def test_config1_every_element_equals_the_model(pkg, oracle, dev, variant):
+    """256 x 512 x 1024 in 2, 3 and 5 partitions: all 131072 outputs are the modelled kernel's bits."""
+    mm = importlib.import_module("oracle.mfma_model")
+    flag = pkg._lib.SPLIT_SUM_IN_KERNEL
+    cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0])
+    ref = oracle.ref_kernel(cpu)
+    idx = np.stack(np.meshgrid(np.arange(256), np.arange(512), indexing="ij"), -1).reshape(-1, 2)
+    for split in (2, 3, 5):
+        out = pkg.custom_kernel(_to(cpu, dev), variant=variant, split_k=split | flag).cpu()
+        want, _ = mm.model_kernel_at(cpu, idx, split)
+        assert torch.equal(_bits(out.reshape(-1)), _bits(want)), "variant %d split %d" % (variant, split)
+        ok, nstrict, nun = oracle.parity_report(out, ref, cpu, split, RTOL, ATOL)
+        assert ok, "variant %d split %d: %d beyond the bar, %d not reproduced" % (variant, split, nstrict, nun)
+
+
+@pytest.mark.parametrize("m,n,k", [(272, 2112, 512), (304, 400, 384), (64, 1024, 1024), (512, 144, 1280), (1, 7, 256), (33, 129, 384),
+                                   (516, 264, 384), (4095, 512, 256), (1021, 264, 1536), (61, 2048, 1024), (3, 18432, 512),
+                                   (257, 192, 384), (513, 136, 1024), (300, 1001, 1280), (1024, 512, 7168), (130, 4100, 1536)])
+def test_ragged_shapes_against_the_oracle_and_the_two_launch_split(pkg, oracle, dev, m, n, k):
+    """Tails in m and n, tiles larger than the matrix, partitions of unequal length (K blocks not a multiple of the
+    split), more workgroups than places on the chip: within the bar of the oracle, and the bits of the same split
+    with the reduce kernel."""
+    flag = pkg._lib.SPLIT_SUM_IN_KERNEL
+    cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[2], m=m, n=n, k=k)
+    ref = oracle.ref_kernel(cpu)
+    data = _to(cpu, dev)
+    for variant in TILED:
+        for split in (2, 3, 4, 7):
+            if split > k // 128:
+                continue
+            two = pkg.custom_kernel(data, variant=variant, split_k=split).clone()
+            data[4].fill_(7.0)
+            one = pkg.custom_kernel(data, variant=variant, split_k=split | flag)
+            assert torch.equal(_bits(one), _bits(two)), "%dx%dx%d variant %d split %d" % (m, n, k, variant, split)
+            ok, nbad, maxerr = oracle.within_tolerance(one, ref, RTOL, ATOL)
+            assert ok, "%dx%dx%d variant %d split %d: %d elements outside the bar (max abs err %g)" % (m, n, k, variant, split, nbad, maxerr)
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 18432, 7168), (1024, 1536, 7168), (6144, 576, 7168), (1, 18432, 7168)])
+def test_what_the_planner_sums_in_the_kernel(pkg, oracle, dev, m, n, k):
+    """Shapes planned with two or three partitions at full size, every element against the oracle, and the bits of
+    the same plan with the reduce kernel."""
+    plan = pkg.plan(m, n, k)
+    assert plan.split_k in (2, 3) and plan.sum_in_kernel == 1
+    cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[3], m=m, n=n, k=k)
+    data = _to(cpu, dev)
+    out = pkg.custom_kernel(data).clone()
+    ok, nstrict, nun = oracle.parity_report(out, oracle.ref_kernel(cpu), cpu, plan.split_k, RTOL, ATOL)
+    assert ok, "%dx%dx%d: %d beyond the bar, %d not reproduced" % (m, n, k, nstrict, nun)
+    two = pkg.custom_kernel(data, variant=plan.variant, split_k=plan.split_k)
+    assert torch.equal(_bits(out), _bits(two))
+
+
+def test_whatever_the_workspace_holds(pkg, dev):
+    """The counters carry the call's tag: zeros, ones, random bytes or the counters of a call that was cut short
+    (here: written by hand) in the head of the workspace all count as `nobody has arrived`."""
+    sub = importlib.import_module("amd-developer-challenge-2025_amd.submission")
+    flag = pkg._lib.SPLIT_SUM_IN_KERNEL
+    cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0])
+    data = _to(cpu, dev)
+    want = pkg.custom_kernel(data, variant=12, split_k=3).clone()
+    need = 16384 + 3 * (256 + 255) * (512 + 255) * 4
+    ws = sub._workspace(dev, need, torch.cuda.current_stream().cuda_stream)
+    gen = torch.Generator(device="cpu").manual_seed(11)
+    fills = [lambda: ws.zero_(), lambda: ws.fill_(255), lambda: ws.copy_(torch.randint(0, 256, (ws.numel(),), generator=gen, dtype=torch.uint8)),
+             lambda: ws[:16384].view(torch.int64).fill_((0x1234567 << 16) | 2)]        # a foreign tag with two arrivals
+    for i, fill in enumerate(fills):
+        fill()
+        data[4].fill_(-3.0)
+        got = pkg.custom_kernel(data, variant=12, split_k=3 | flag)
+        torch.cuda.synchronize()
+        assert torch.equal(_bits(got), _bits(want)), "fill %d" % i
+    # after a call every counter that was used is back at zero
+    ws.zero_()
+    pkg.custom_kernel(data, variant=12, split_k=3 | flag)
+    torch.cuda.synchronize()
+    assert int(ws[256:16384].view(torch.int64).ne(0).sum()) == 0
+
+
+def test_repeated_calls_and_graph_replays(pkg, dev):
+    """A replay of a captured launch carries the same tag as the first run: the last workgroup of every tile puts
+    the counter back to zero, so every replay starts clean."""
+    flag = pkg._lib.SPLIT_SUM_IN_KERNEL
+    cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[3], m=64, n=2304, k=2048)
+    data = _to(cpu, dev)
+    first = pkg.custom_kernel(data, variant=12, split_k=3).clone()
+    for _ in range(3):
+        data[4].fill_(5.0)
+        assert torch.equal(_bits(pkg.custom_kernel(data, variant=12, split_k=3 | flag)), _bits(first))
+    other = _to(pkg.inputs.make_dense(pkg.inputs.CONFIGS[2], m=64, n=2304, k=2048), dev)
+    want_other = pkg.custom_kernel(other, variant=12, split_k=3).clone()
+    static = tuple(t.clone() for t in data)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        pkg.custom_kernel(static, variant=12, split_k=3 | flag)  # the capture stream's workspace exists from here on
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        pkg.custom_kernel(static, variant=12, split_k=3 | flag)
+    for rep in range(4):
+        src, want = (data, first) if rep % 2 == 0 else (other, want_other)
+        for dst, s in zip(static[:4], src[:4]):
+            dst.copy_(s)
+        static[4].fill_(3.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(_bits(static[4]), _bits(want)), "replay %d" % rep
+        pkg.custom_kernel(data)                                  # eager work between replays
+        torch.cuda.synchronize()
+
+
+def test_more_tiles_than_counters_takes_the_reduce_kernel(pkg, oracle, dev):
+    """4096 tiles of 64 x 128 are more than the workspace's head has counters for: the call takes the two-launch
+    form and gives the same bits."""
+    flag = pkg._lib.SPLIT_SUM_IN_KERNEL
+    cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[2], m=4096, n=8192, k=512)
+    data = _to(cpu, dev)
+    two = pkg.custom_kernel(data, variant=4, split_k=2).clone()
+    data[4].fill_(1.0)
+    one = pkg.custom_kernel(data, variant=4, split_k=2 | flag)
+    assert torch.equal(_bits(one), _bits(two))
+
+
+def test_workspace_too_small_and_kernels_without_the_sum(pkg, dev):
+    lib = pkg._lib.load()
+    flag = pkg._lib.SPLIT_SUM_IN_KERNEL
+    cpu = pkg.inputs.make_dense(pkg.inputs.CONFIGS[0])
+    a, b, sa, sb, c = _to(cpu, dev)
+    need = 16384 + 2 * 3 * 256 * 256 * 4                         # 2 tiles of 256 x 256, three partitions
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    args = (a.data_ptr(), b.data_ptr(), sa.data_ptr(), sb.data_ptr(), c.data_ptr())
+    assert lib.fp8bs_gemm_ex(*args, ws.data_ptr(), need - 1, 256, 512, 1024, 2, 3 | flag, None) == 3      # FP8BS_ERR_WORKSPACE
+    assert lib.fp8bs_gemm_ex(*args, None, 0, 256, 512, 1024, 2, 3 | flag, None) == 3
+    assert lib.fp8bs_gemm_ex(*args, ws.data_ptr(), need, 256, 512, 1024, 2, 3 | flag, None) == 0
+    torch.cuda.synchronize()
+    for variant in (1, 6):                                       # the scalar and the streaming kernels have no such sum
+        assert lib.fp8bs_gemm_ex(*args, ws.data_ptr(), need, 256, 512, 1024, variant, 3 | flag, None) == 7   # FP8BS_ERR_BAD_VARIANT
