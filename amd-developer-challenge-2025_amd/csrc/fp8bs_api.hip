@@ -186,7 +186,7 @@ void choose_skinny(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may
     if (num_cus <= 0) num_cus = 256;
     const int kbt = k / KBLK;
     const long tiles = cdiv(m, 64) * cdiv(n, 256);
-    int best_s = 1; double best = 0;
+    int best_s = 1; double best = 0; bool best_fused = false;
     for (int s = 1; s <= 8 && s <= kbt; s++) {
         if (s > 1 && !may_split) break;
         const long wgs = tiles * s;
@@ -195,12 +195,17 @@ void choose_skinny(int m, int n, int k, int num_cus, fp8bs_plan_t* out, bool may
         if (t_block < 1.05) t_block = 1.05;
         double cost = (double)cdiv(wgs, num_cus) * (2.0 + (double)cdiv(kbt, s) * t_block);
         if (s > 1) cost += 4.0 + 0.24 * s + 1.19e-6 * s * (double)m * (double)n;
-        // two or three partitions are summed in the kernel (64 x 18432 x 7168, b from HBM: 33.5 us against 34.4 with
-        // three, 37.4 against 38.6 with two; with four 52.8 against 49.6)
-        if (s == 2 || s == 3) cost -= 0.8;
-        if (s == 1 || cost < best) { best = cost; best_s = s; }
+        // Two or three partitions in one round of workgroups are summed in the kernel where the planes are large
+        // enough for the reduce launch to cost more than the chain of round trips that replaces it (the partial
+        // tile's acknowledged stores, the count, the last workgroup's reads).  b from HBM, three partitions of
+        // 18432 x 7168: 64 rows 33.7 us against 34.4 with the reduce launch, 16 rows 30.3 against 29.3, one row 31.0
+        // against 29.0; two partitions of 64 rows 37.4 against 38.6, four 52.8 against 49.6.
+        const double in_kernel = 2.05 - 0.78e-6 * s * (double)m * (double)n;
+        const bool fuse = (s == 2 || s == 3) && wgs <= num_cus && in_kernel < 0 && can_sum_in_kernel(m, n, FP8BS_VARIANT_T64x256S3, s);
+        if (fuse) cost += in_kernel;
+        if (s == 1 || cost < best) { best = cost; best_s = s; best_fused = fuse; }
     }
-    fill_plan(m, n, k, FP8BS_VARIANT_T64x256S3, best_s, out, 0, best_s == 2 || best_s == 3);
+    fill_plan(m, n, k, FP8BS_VARIANT_T64x256S3, best_s, out, 0, best_fused);
 }
 
 // Shape-family rule.  A few rows against a large b -> the 64 x 256 three-stage tile.  Everything else -> the

@@ -940,13 +940,24 @@ void gemm_tr_kernel(const GemmArgs p) {
         // (the counter is read ahead of the stores: the value only seeds the exchange below, which finds out if it is stale)
         unsigned long long seen = 0;
         if (tid == 0) seen = __hip_atomic_load(&counters[sk_first], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // Lanes whose row or columns lie outside the matrix neither store nor load their piece (an offset beyond the
+        // slot drops a store and makes a load return zeros): one row against 18432 columns leaves 1 KB per workgroup
+        // in the workspace instead of 32 KB (31.6 us with every lane storing, against 29.1 as two launches).
+        uint32_t rows_in = 0, cols_in = 0;                 // bit t: the lane's row of m tile t exists; bit u: its columns of n tile u
+#pragma unroll
+        for (int t = 0; t < C::MT; t++) rows_in |= (m0 + wave_m * WM + 16 * t + i16 < row_hi ? 1u : 0u) << t;
+#pragma unroll
+        for (int u = 0; u < C::NT; u++) cols_in |= (n0 + wave_n * WN + 16 * u + 4 * g < p.n ? 1u : 0u) << u;
+        auto piece = [&](int x) -> uint32_t {               // x = t * NT + u, a compile-time number at every use
+            return ((rows_in >> (x / C::NT)) & (cols_in >> (x % C::NT)) & 1u) ? voff + (uint32_t)x * 1024u : 0xFFFFFFFFu;
+        };
         if (wave_active) {
             __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(tile_slots + (size_t)split_z * SLOT_BYTES), 0, SLOT_BYTES, 0x00020000);
 #pragma unroll
             for (int t = 0; t < C::MT; t++)
 #pragma unroll
                 for (int u = 0; u < C::NT; u++)
-                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, acc[t][u]), rs, voff + (uint32_t)(t * C::NT + u) * 1024u, 0, AUX_AGENT);
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, acc[t][u]), rs, piece(t * C::NT + u), 0, AUX_AGENT);
         }
         wait_vmcnt<0>();                                    // acknowledged from the agent's point of coherence
         __syncthreads();
@@ -964,7 +975,7 @@ void gemm_tr_kernel(const GemmArgs p) {
         __syncthreads();
         store_output = __builtin_amdgcn_readfirstlane(last_in) != 0;
         if (store_output && wave_active) {
-            __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)tile_slots, 0, (uint32_t)p.split_k * SLOT_BYTES, 0x00020000);
+            auto slot_of = [&](int z) { return __builtin_amdgcn_make_buffer_rsrc((void*)(tile_slots + (size_t)z * SLOT_BYTES), 0, SLOT_BYTES, 0x00020000); };
             // S partitions known at compile time: the loads of all other partitions' pieces of a batch are in flight
             // together (up to 16 of 16 bytes per lane); S = 0: any number, one partition at a time
             [[maybe_unused]] auto sum_planes = [&]<int S>() {
@@ -977,10 +988,10 @@ void gemm_tr_kernel(const GemmArgs p) {
                         v4f part[S - 1][BATCH];                              // the other partitions, ascending
 #pragma unroll
                         for (int j = 0; j < S - 1; j++) {
-                            const uint32_t soff = (uint32_t)(j + (j >= split_z ? 1 : 0)) * SLOT_BYTES;
+                            __amdgpu_buffer_rsrc_t rs = slot_of(j + (j >= split_z ? 1 : 0));
 #pragma unroll
                             for (int i = 0; i < BATCH; i++)
-                                part[j][i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff + (uint32_t)(base + i) * 1024u, AUX_AGENT));
+                                part[j][i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs, piece(base + i), 0, AUX_AGENT));
                         }
 #pragma unroll
                         for (int i = 0; i < BATCH; i++) {
@@ -1003,9 +1014,10 @@ void gemm_tr_kernel(const GemmArgs p) {
 #pragma unroll
                                 for (int i = 0; i < BATCH; i++) part[i] = acc[(base + i) / C::NT][(base + i) % C::NT];
                             } else {
+                                __amdgpu_buffer_rsrc_t rs = slot_of(z);
 #pragma unroll
                                 for (int i = 0; i < BATCH; i++)
-                                    part[i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs, voff, (uint32_t)z * SLOT_BYTES + (uint32_t)(base + i) * 1024u, AUX_AGENT));
+                                    part[i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs, piece(base + i), 0, AUX_AGENT));
                             }
 #pragma unroll
                             for (int i = 0; i < BATCH; i++) sum[i] = z == 0 ? part[i] : sum[i] + part[i];
@@ -1028,9 +1040,10 @@ void gemm_tr_kernel(const GemmArgs p) {
 #pragma unroll
                             for (int i = 0; i < GB; i++) part[i] = acc[(base + i) / C::NT][(base + i) % C::NT];
                         } else {
+                            __amdgpu_buffer_rsrc_t rs = slot_of(z);
 #pragma unroll
                             for (int i = 0; i < GB; i++)
-                                part[i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs, voff, (uint32_t)z * SLOT_BYTES + (uint32_t)(base + i) * 1024u, AUX_AGENT));
+                                part[i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs, piece(base + i), 0, AUX_AGENT));
                         }
 #pragma unroll
                         for (int i = 0; i < GB; i++) sum[i] = z == 0 ? part[i] : sum[i] + part[i];

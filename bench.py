@@ -407,7 +407,7 @@ def main():
         us, us_min = time_calls(lambda i: pkg.custom_kernel(sets[i % nsets]), args.steps, args.warmup)
         per_config[dcfg.name] = {"us": round(us, 2), "us_min": round(us_min, 2), "gbs": round(by / us * 1e-3, 1), "bytes": by,
                                  "input_sets": nsets, "bound": "hbm", "frac": round(by / us * 1e-3 / PEAK_HBM_GBS, 4),
-                                 "note": "one row against configuration 4's weights: the planner's tile with its K split, then the reduction"}
+                                 "note": "one row against configuration 4's weights: the planner's tile with its K split and the reduce launch (planes this small are cheaper to sum there than in the kernel)"}
         sets = None
     # ---- configuration 2 one row and one column short: rows of a, b and c that start on odd bytes ----
     if 2 in wanted or 3 in wanted:

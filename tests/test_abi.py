@@ -76,7 +76,7 @@ def test_plan_shape_families(pkg):
         assert p.variant == q.variant and p.variant not in (1, 6, 7, 8) and p.split_k == q.split_k
         assert p.workspace_bytes == _planned_workspace(p, m, 192)
     p, q = pkg.plan(3, 18432, 7168), pkg.plan(4, 18432, 7168) # a few rows against a large b: the same skinny plan for any m
-    assert p.variant == q.variant == 12 and p.split_k == q.split_k and p.workspace_bytes == q.workspace_bytes == _planned_workspace(p, 3, 18432)
+    assert p.variant == q.variant == 12 and p.split_k == q.split_k and p.workspace_bytes == _planned_workspace(p, 3, 18432) and q.workspace_bytes == _planned_workspace(q, 4, 18432)
     assert pkg.plan(3, 190, 256).variant in (3, 4, 12)
     p = pkg.plan(256, 512, 1024)                        # small: one of the sub-256 tiles, never the scalar kernel
     assert p.variant in (3, 4, 10, 12) and p.split_k >= 1 and p.split_k <= 8
@@ -105,8 +105,10 @@ def test_plan_skinny_rule_and_the_streaming_kernels(pkg):
             assert p.variant == 12 and p.grid_x == -(-n // 256) * p.split_k, (m, n, k, p.variant)
         assert p.variant not in (1, 6, 7, 8)
         assert 1 <= p.split_k <= 8 and p.workspace_bytes == _planned_workspace(p, m, n)
-        assert p.sum_in_kernel == (1 if p.split_k in (2, 3) else 0)     # two or three partitions are summed in the kernel
+        assert p.sum_in_kernel == 0 or p.split_k in (2, 3)              # only two or three partitions are summed in the kernel
     assert pkg.plan(1536, 1536, 4096).variant == 12           # the cost model's pick for a few hundred rows per tile column
+    # few rows: summed in the kernel only where the planes are large enough for the reduce launch to cost more
+    assert pkg.plan(64, 18432, 7168).sum_in_kernel == 1 and pkg.plan(1, 18432, 7168).sum_in_kernel == 0
     for m in (1, 5, 63):                                      # rows that are not a multiple of four: the same plan
         p, q = pkg.plan(m, 18432, 7168), pkg.plan((m + 3) & ~3, 18432, 7168)
         assert p.variant == q.variant == 12 and p.split_k == q.split_k
