@@ -1029,7 +1029,8 @@ void gemm_tr_kernel(const GemmArgs p) {
                 }
             };
             if constexpr (NG > 16) {
-                // 72 to 128 accumulator registers leave room for one partition's batch of three or four
+                // 72 to 128 accumulator registers leave room for one partition's batch of three or four (the loop of
+                // the S = 0 case above, written out: called through the lambda it cost the 256x256 tile ~40 spilled registers)
                 constexpr int GB = NG % 4 == 0 ? 4 : (NG % 3 == 0 ? 3 : (NG % 2 == 0 ? 2 : 1));
 #pragma unroll
                 for (int base = 0; base < NG; base += GB) {
