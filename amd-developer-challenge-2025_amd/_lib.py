@@ -33,6 +33,7 @@ class Plan(ctypes.Structure):
 
 
 SPLIT_SUM_IN_KERNEL = 1 << 30        # FP8BS_SPLIT_SUM_IN_KERNEL
+MIN_VERSION = 300                    # fp8bs_version() of the first library whose fp8bs_plan_t has sum_in_kernel
 
 
 _lib = None
@@ -51,6 +52,10 @@ def load() -> ctypes.CDLL:
     vp, i32, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
     lib.fp8bs_version.restype = i32
     lib.fp8bs_version.argtypes = []
+    if lib.fp8bs_version() < MIN_VERSION:
+        # an older build fills a shorter fp8bs_plan_t than the Plan mirrored here
+        raise RuntimeError("%s is version %d, this package needs %d or later: rebuild it with "
+                           "`python amd-developer-challenge-2025_amd/build.py`" % (LIB_PATH, lib.fp8bs_version(), MIN_VERSION))
     lib.fp8bs_strerror.restype = ctypes.c_char_p
     lib.fp8bs_strerror.argtypes = [i32]
     lib.fp8bs_plan.restype = i32

@@ -291,7 +291,7 @@ static int scratch_address(void** out, hipStream_t stream) {
 
 extern "C" {
 
-int fp8bs_version(void) { return 100; }
+int fp8bs_version(void) { return 300; }      // 0.3.0: fp8bs_plan_t grew (sum_in_kernel)
 
 const char* fp8bs_strerror(int status) {
     switch (status) {

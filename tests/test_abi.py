@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol(pkg):
     assert set(declared) == set(pkg._lib.EXPORTS)
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.fp8bs_version() >= 100
+    assert lib.fp8bs_version() >= pkg._lib.MIN_VERSION
 
 
 def test_every_variant_has_a_name_and_the_plan_struct_matches_the_header(pkg):
