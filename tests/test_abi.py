@@ -34,6 +34,9 @@ def test_every_variant_has_a_name_and_the_plan_struct_matches_the_header(pkg):
     body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
     fields = [f.strip() for decl in re.findall(r"(?:int32_t|uint64_t)\s+([^;]+);", body) for f in decl.split(",")]
     assert fields == [name for name, _ in pkg._lib.Plan._fields_]
+    shift = int(re.search(r"#define FP8BS_SPLIT_SUM_IN_KERNEL \(1 << (\d+)\)", text).group(1))
+    assert pkg._lib.SPLIT_SUM_IN_KERNEL == 1 << shift
+    assert ctypes.sizeof(pkg._lib.Plan) == 4 * 12 + 8                # twelve int32, then the 8-byte workspace size
 
 
 def test_plan_with_the_devices_cu_count(pkg):
